@@ -1,0 +1,188 @@
+/*
+ * sparseops_hip.h -- C ABI of libsparseops_hip.so, the MI355X (gfx950) device side
+ * of the ELLPACK compute path.
+ *
+ * The reference is a CPU library whose consumers are C++ callers of its headers
+ * and Python through pybind11; it has no FFI of its own.  This header is the
+ * boundary a maintainer binds instead of the reference's CPU kernels: plain C,
+ * opaque handles, caller-owned pointers and sizes, no C++ or torch types.  Each
+ * entry point cites the reference interface it stands in for.
+ *
+ * Conventions
+ *   - every function returns so_status (0 = ok) and never throws or aborts;
+ *     so_last_error() gives the message of the calling thread's last failure.
+ *   - "d" parameters are device pointers obtained from so_malloc (or any HIP
+ *     allocation on the context's device); all others are host pointers.
+ *   - every launch goes to the context's single stream; calls return without
+ *     waiting for the device unless stated (so_d2h, so_sync, so_timer_end wait).
+ *   - matrices are row-major; activations of the layer chain are
+ *     [features x B] with the batch contiguous (include/sparse_onnx.hpp:148-154),
+ *     4-D tensors are [C][H][W][B] (src/layers/conv_kernels.cpp:342-347).
+ *   - all arithmetic is fp32; every output element is produced by the same
+ *     rounding sequence as the reference (bias first, then one fused
+ *     multiply-add per stored nonzero in ascending slot order), except so_matvec
+ *     whose in-row summation order differs (wave reduction) and is accurate to
+ *     fp32 round-off.
+ */
+#ifndef SPARSEOPS_HIP_H
+#define SPARSEOPS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int so_status;
+enum {
+    SO_OK = 0,
+    SO_ERR_NO_DEVICE = 1, /* no usable HIP device / HIP runtime failed to initialise */
+    SO_ERR_INVALID = 2,   /* bad argument (null pointer, shape mismatch, bad enum) */
+    SO_ERR_OOM = 3,       /* device or host allocation failed */
+    SO_ERR_HIP = 4,       /* a HIP call failed; message holds hipGetErrorString */
+    SO_ERR_BOUNDS = 5     /* ELLPACK content invalid: idx >= n or nnz > r */
+};
+
+/* Fused epilogue of so_matmul / so_conv2d.  NONE and RELU are the reference's
+ * template flag FUSE_RELU (src/ellpack_matmul.cpp:68-70); SIGMOID and TANH equal
+ * the reference's separate activation layers applied to the matmul result
+ * (src/layers/activation.cpp:38-40, 58-60). */
+enum { SO_ACT_NONE = 0, SO_ACT_RELU = 1, SO_ACT_SIGMOID = 2, SO_ACT_TANH = 3 };
+
+/* Device layouts kept for an uploaded ELLPACK matrix (bit flags).
+ * ROW  : Wd[i*r + k], idx[i*r + k]  -- the encoder's own layout
+ *        (include/ellpack_encoder.hpp:6-23); used by so_matmul / so_conv2d and
+ *        by so_matvec for long rows.
+ * SLOT : WdT[k*m + i], idxT[k*m + i] -- slot-major transpose so that the k-th
+ *        nonzeros of consecutive rows are contiguous; used by so_matvec when
+ *        one lane owns one row.
+ * BINS : rows grouped by nnz into length classes for so_matvec on skewed
+ *        matrices, so padding is never streamed. */
+enum { SO_LAYOUT_ROW = 1, SO_LAYOUT_SLOT = 2, SO_LAYOUT_BINS = 4 };
+
+typedef struct so_ctx so_ctx;         /* one device + one stream + staging arena */
+typedef struct so_ellpack so_ellpack; /* device-resident ELLPACK matrix */
+
+/* Geometry of one convolution as the reference's loader derives it
+ * (ConvAttr, include/sparse_onnx.hpp:66-98; src/sparse_onnx.cpp:408-451).
+ * Column k of the Cout x K weight matrix is (cin, kh, kw) with kw fastest. */
+typedef struct {
+    uint32_t Cin, Cout, kH, kW;
+    uint32_t stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
+    uint32_t H_in, W_in, H_out, W_out;
+} so_conv_geom;
+
+/* PoolAttr (include/sparse_onnx.hpp:101-112). */
+typedef struct {
+    uint32_t C, H, W, H_out, W_out;
+    int32_t kH, kW, sH, sW, padH0, padW0;
+} so_pool_geom;
+
+/* ---- runtime ------------------------------------------------------------- */
+
+/* Number of HIP devices; SO_ERR_NO_DEVICE (and *n = 0) when there is none. */
+so_status so_device_count(int *n);
+/* Create a context on `device` (its own non-blocking stream, default priority). */
+so_status so_init(int device, so_ctx **out);
+so_status so_destroy(so_ctx *ctx);
+/* Message of the last failure on the calling thread ("" if none). */
+const char *so_last_error(void);
+/* Device name and compute-unit count of the context's device. */
+so_status so_device_info(so_ctx *ctx, char *name, size_t name_len, int *compute_units);
+
+so_status so_malloc(so_ctx *ctx, size_t bytes, void **dptr);
+so_status so_free(so_ctx *ctx, void *dptr);
+so_status so_h2d(so_ctx *ctx, void *dst, const void *src, size_t bytes); /* waits */
+so_status so_d2h(so_ctx *ctx, void *dst, const void *src, size_t bytes); /* waits */
+so_status so_d2d(so_ctx *ctx, void *dst, const void *src, size_t bytes);
+so_status so_fill_zero(so_ctx *ctx, void *dptr, size_t bytes); /* fill kernel, graph-safe */
+so_status so_sync(so_ctx *ctx);
+
+/* HIP-event stopwatch on the context's stream: begin records an event, end
+ * records a second one, waits for it and returns the elapsed milliseconds. */
+so_status so_timer_begin(so_ctx *ctx);
+so_status so_timer_end(so_ctx *ctx, float *ms);
+
+/* ---- ELLPACK on the device ---------------------------------------------- */
+
+/* Upload the encoder's arrays once (struct Ellpack, include/ellpack_encoder.hpp:6-23:
+ * Wd[m*r], idx[m*r], nnz[m]).  Validates nnz[i] <= r and idx < n for every stored
+ * slot (the reference validates only in a benchmark,
+ * benchmark-mkl/matvec/bench_matvec.cpp:83-98) and fails with SO_ERR_BOUNDS.
+ * `layouts` is a mask of SO_LAYOUT_*; ROW is always kept.  m, n or r may be 0. */
+so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint32_t *idx,
+                            const uint32_t *nnz, uint32_t m, uint32_t n, uint32_t r,
+                            int layouts, so_ellpack **out);
+so_status so_ellpack_free(so_ctx *ctx, so_ellpack *E);
+so_status so_ellpack_dims(const so_ellpack *E, uint32_t *m, uint32_t *n, uint32_t *r,
+                          uint64_t *total_nnz, int *layouts);
+/* Read the device copy back, for the bit-exact layout check.  layout = ROW
+ * returns Wd/idx as uploaded; layout = SLOT returns the slot-major arrays
+ * (WdT[k*m+i]); nnz may be NULL. */
+so_status so_ellpack_download(so_ctx *ctx, const so_ellpack *E, int layout,
+                              float *Wd, uint32_t *idx, uint32_t *nnz);
+
+/* ---- kernels ------------------------------------------------------------ */
+
+/* Y[m x C] = act(E * X[n x C] + bias): ellpack_matmul_fused<USE_MASK,FUSE_RELU>
+ * (src/ellpack_matmul.cpp:11-92) and its dispatcher ellpack_matmul
+ * (include/ellpack_matmul.hpp:23-43).  dBias may be NULL (zero start). */
+so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
+                    const float *dBias, float *dY, int act);
+
+/* y[m] = E * x[n] + bias: ellpack_matvec (src/ellpack_matvec.cpp:20-147).
+ * `layout` picks the kernel: SO_LAYOUT_ROW (one wave per row), SO_LAYOUT_SLOT
+ * (one lane per row on the slot-major copy), SO_LAYOUT_BINS (length classes),
+ * or 0 to let the library choose from what was uploaded. */
+so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx,
+                    const float *dBias, float *dy, int layout);
+
+/* Per-layer convolution plan, built once at load time: for every stored nonzero
+ * of E (Cout x Cin*kH*kW) the input offset and (dh, dw) of its tap -- the role of
+ * the reference's kmap (src/sparse_onnx.cpp:440-451); the (ho, wo, b)-dependent
+ * part of the patch index is generated inside the kernel, so there is no
+ * patch_indices table (src/sparse_onnx.cpp:476-497).  E must outlive the plan.
+ * Checks H_out/W_out against the loader's formula (src/sparse_onnx.cpp:428-429). */
+typedef struct so_conv_plan so_conv_plan;
+so_status so_conv_plan_create(so_ctx *ctx, const so_ellpack *E, const so_conv_geom *g,
+                              so_conv_plan **out);
+so_status so_conv_plan_free(so_ctx *ctx, so_conv_plan *plan);
+
+/* Sparse convolution by implicit im2col: conv2d_implicit_im2col_fmajor
+ * (src/layers/conv.cpp:16-108), on the [C][H][W][B] layout of
+ * conv2d_patchmajor_tiled (src/layers/conv_kernels.cpp:342-470), which is what
+ * applyConv runs (src/layers/conv.cpp:118-135).  dX is [Cin][H_in][W_in][B],
+ * dY is [Cout][H_out][W_out][B]; dBias may be NULL. */
+so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B,
+                    const float *dBias, float *dY, int act);
+
+/* applyMaxPool / applyGlobalAveragePool (src/layers/pool.cpp:28-101, 103-154)
+ * on [C][H][W][B]; GAP writes [C][B]. */
+so_status so_maxpool(so_ctx *ctx, const so_pool_geom *p, const float *dX, uint32_t B, float *dY);
+so_status so_gap(so_ctx *ctx, uint32_t C, uint32_t H, uint32_t W, const float *dX,
+                 uint32_t B, float *dY);
+/* applyAdd (src/layers/add.cpp:9-76): D = A + B over len floats (D may alias A or B). */
+so_status so_add(so_ctx *ctx, const float *dA, const float *dB, size_t len, float *dD);
+/* applyRelu / applySigmoid / applyTanh (src/layers/activation.cpp:3-62). */
+so_status so_act(so_ctx *ctx, int act, const float *dX, size_t len, float *dY);
+/* dst[cols x rows] = transpose of src[rows x cols]; converts a C-order (B, F)
+ * array to the kernels' [F x B] layout and back (the reference's Python tests
+ * do this on the host with Fortran-order arrays, tests/full_test.py:77-88). */
+so_status so_transpose(so_ctx *ctx, const float *dSrc, uint32_t rows, uint32_t cols, float *dDst);
+
+/* ---- launch graphs -------------------------------------------------------
+ * Record every launch made on the context between begin and end into one
+ * hipGraph, then replay it with a single submission (SparseOnnxModel::run uses
+ * this for the layer chain, src/model_run.cpp:28-127).  No allocation, copy to
+ * or from the host, or timer call may happen while recording. */
+typedef struct so_graph so_graph;
+so_status so_graph_begin(so_ctx *ctx);
+so_status so_graph_end(so_ctx *ctx, so_graph **out);
+so_status so_graph_launch(so_ctx *ctx, so_graph *g);
+so_status so_graph_free(so_ctx *ctx, so_graph *g);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPARSEOPS_HIP_H */

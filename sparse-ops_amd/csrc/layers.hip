@@ -1,0 +1,165 @@
+// Bandwidth-bound layer kernels of the model chain: max-pool, global average
+// pool, elementwise add, stand-alone activations and the 2-D transpose used at
+// the host boundary.  All tensors are [C][H][W][B] / [features][B], batch innermost,
+// so consecutive lanes always touch consecutive addresses.
+#include "so_internal.h"
+
+#include <algorithm>
+
+namespace {
+
+constexpr int kBlock = 256;
+
+// applyMaxPool (src/layers/pool.cpp:28-101): -inf start, taps outside the image skipped.
+__global__ __launch_bounds__(kBlock)
+void maxpool_kernel(so_pool_geom p, const float *__restrict__ X, uint32_t B, uint64_t total,
+                    float *__restrict__ Y)
+{
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (uint64_t q = (uint64_t)blockIdx.x * kBlock + threadIdx.x; q < total; q += stride) {
+        const uint32_t b = (uint32_t)(q % B);
+        uint64_t t = q / B;
+        const uint32_t wo = (uint32_t)(t % p.W_out); t /= p.W_out;
+        const uint32_t ho = (uint32_t)(t % p.H_out);
+        const uint32_t c = (uint32_t)(t / p.H_out);
+        const int32_t h0 = (int32_t)ho * p.sH - p.padH0, w0 = (int32_t)wo * p.sW - p.padW0;
+        float v = -INFINITY;
+        for (int32_t kh = 0; kh < p.kH; ++kh) {
+            const int32_t hin = h0 + kh;
+            if ((uint32_t)hin >= p.H) continue;
+            for (int32_t kw = 0; kw < p.kW; ++kw) {
+                const int32_t win = w0 + kw;
+                if ((uint32_t)win >= p.W) continue;
+                const float x = X[(((uint64_t)c * p.H + (uint32_t)hin) * p.W + (uint32_t)win) * B + b];
+                v = x > v ? x : v;
+            }
+        }
+        Y[q] = v;
+    }
+}
+
+// applyGlobalAveragePool (src/layers/pool.cpp:103-154): fp32 running sum over h
+// then w, times 1.0f/float(H*W).  One lane per (c, b).
+__global__ __launch_bounds__(kBlock)
+void gap_kernel(uint32_t C, uint32_t HW, const float *__restrict__ X, uint32_t B, float scale,
+                float *__restrict__ Y)
+{
+    const uint64_t total = (uint64_t)C * B;
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (uint64_t q = (uint64_t)blockIdx.x * kBlock + threadIdx.x; q < total; q += stride) {
+        const uint32_t b = (uint32_t)(q % B);
+        const uint64_t c = q / B;
+        const float *xp = X + c * HW * B + b;
+        float s = 0.0f;
+        for (uint32_t i = 0; i < HW; ++i) s = s + xp[(uint64_t)i * B];
+        Y[q] = s * scale;
+    }
+}
+
+__global__ __launch_bounds__(kBlock)
+void add_kernel(const float *__restrict__ A, const float *__restrict__ Bv, size_t len, float *D)
+{
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < len; i += stride) D[i] = A[i] + Bv[i];
+}
+
+template <int ACT>
+__global__ __launch_bounds__(kBlock)
+void act_kernel(const float *X, size_t len, float *Y)
+{
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < len; i += stride)
+        Y[i] = so_epilogue<ACT>(X[i]);
+}
+
+// 64x64 tiles through LDS (+1 padding against bank conflicts): both the read of
+// src rows and the write of dst rows are coalesced.
+__global__ __launch_bounds__(kBlock)
+void transpose_kernel(const float *__restrict__ src, uint32_t rows, uint32_t cols, float *__restrict__ dst)
+{
+    __shared__ float tile[64][65];
+    const uint32_t tx = threadIdx.x & 63u, ty = threadIdx.x >> 6;  // 64 x 4
+    const uint32_t r0 = blockIdx.y * 64u, c0 = blockIdx.x * 64u;
+    for (uint32_t i = ty; i < 64; i += 4)
+        if (r0 + i < rows && c0 + tx < cols) tile[i][tx] = src[(size_t)(r0 + i) * cols + c0 + tx];
+    __syncthreads();
+    for (uint32_t i = ty; i < 64; i += 4)
+        if (c0 + i < cols && r0 + tx < rows) dst[(size_t)(c0 + i) * rows + r0 + tx] = tile[tx][i];
+}
+
+uint32_t blocks_for(const so_ctx *ctx, uint64_t work)
+{
+    const uint64_t need = (work + kBlock - 1) / kBlock;
+    return (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>(need, (uint64_t)ctx->compute_units * 16));
+}
+
+} // namespace
+
+extern "C" so_status so_maxpool(so_ctx *ctx, const so_pool_geom *p, const float *dX, uint32_t B, float *dY)
+{
+    SO_REQUIRE(ctx && p, "so_maxpool: null argument");
+    SO_REQUIRE(p->kH > 0 && p->kW > 0 && p->sH > 0 && p->sW > 0 && p->padH0 >= 0 && p->padW0 >= 0,
+               "so_maxpool: kernel and stride must be positive, pads non-negative");
+    const uint64_t total = (uint64_t)p->C * p->H_out * p->W_out * B;
+    if (total == 0) return SO_OK;
+    SO_REQUIRE(dX && dY, "so_maxpool: null tensor");
+    // Every output window must start inside the padded image.
+    SO_REQUIRE((uint64_t)(p->H_out - 1) * p->sH < (uint64_t)p->H + p->padH0 &&
+               (uint64_t)(p->W_out - 1) * p->sW < (uint64_t)p->W + p->padW0,
+               "so_maxpool: output size does not fit the input");
+    maxpool_kernel<<<blocks_for(ctx, total), kBlock, 0, ctx->stream>>>(*p, dX, B, total, dY);
+    SO_LAUNCH_CHECK();
+    return SO_OK;
+}
+
+extern "C" so_status so_gap(so_ctx *ctx, uint32_t C, uint32_t H, uint32_t W, const float *dX,
+                            uint32_t B, float *dY)
+{
+    SO_REQUIRE(ctx != nullptr, "so_gap: ctx is null");
+    const uint64_t total = (uint64_t)C * B;
+    if (total == 0) return SO_OK;
+    SO_REQUIRE(dX && dY && H && W, "so_gap: null tensor or empty plane");
+    const float scale = 1.0f / (float)(H * W);
+    gap_kernel<<<blocks_for(ctx, total), kBlock, 0, ctx->stream>>>(C, H * W, dX, B, scale, dY);
+    SO_LAUNCH_CHECK();
+    return SO_OK;
+}
+
+extern "C" so_status so_add(so_ctx *ctx, const float *dA, const float *dB, size_t len, float *dD)
+{
+    SO_REQUIRE(ctx != nullptr, "so_add: ctx is null");
+    if (len == 0) return SO_OK;
+    SO_REQUIRE(dA && dB && dD, "so_add: null tensor");
+    add_kernel<<<blocks_for(ctx, len), kBlock, 0, ctx->stream>>>(dA, dB, len, dD);
+    SO_LAUNCH_CHECK();
+    return SO_OK;
+}
+
+extern "C" so_status so_act(so_ctx *ctx, int act, const float *dX, size_t len, float *dY)
+{
+    SO_REQUIRE(ctx != nullptr, "so_act: ctx is null");
+    SO_REQUIRE(act >= SO_ACT_NONE && act <= SO_ACT_TANH, "so_act: unknown activation %d", act);
+    if (len == 0) return SO_OK;
+    SO_REQUIRE(dX && dY, "so_act: null tensor");
+    const uint32_t blocks = blocks_for(ctx, len);
+    switch (act) {
+    case SO_ACT_RELU:    act_kernel<SO_ACT_RELU><<<blocks, kBlock, 0, ctx->stream>>>(dX, len, dY); break;
+    case SO_ACT_SIGMOID: act_kernel<SO_ACT_SIGMOID><<<blocks, kBlock, 0, ctx->stream>>>(dX, len, dY); break;
+    case SO_ACT_TANH:    act_kernel<SO_ACT_TANH><<<blocks, kBlock, 0, ctx->stream>>>(dX, len, dY); break;
+    default:             act_kernel<SO_ACT_NONE><<<blocks, kBlock, 0, ctx->stream>>>(dX, len, dY); break;
+    }
+    SO_LAUNCH_CHECK();
+    return SO_OK;
+}
+
+extern "C" so_status so_transpose(so_ctx *ctx, const float *dSrc, uint32_t rows, uint32_t cols, float *dDst)
+{
+    SO_REQUIRE(ctx != nullptr, "so_transpose: ctx is null");
+    if (rows == 0 || cols == 0) return SO_OK;
+    SO_REQUIRE(dSrc && dDst && dSrc != dDst, "so_transpose: null or aliased tensor");
+    const dim3 grid(so_ceil_div(cols, 64), so_ceil_div(rows, 64));
+    SO_REQUIRE(grid.y < 65536, "so_transpose: too many rows");
+    transpose_kernel<<<grid, kBlock, 0, ctx->stream>>>(dSrc, rows, cols, dDst);
+    SO_LAUNCH_CHECK();
+    return SO_OK;
+}

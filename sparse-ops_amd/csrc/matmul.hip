@@ -1,0 +1,177 @@
+// so_matmul: Y[m x C] = act(E * X[n x C] + bias) on gfx950.
+//
+// One wavefront owns one ELLPACK row and one tile of 64*VEC dense columns.  The
+// row's weights and column indices are wave-uniform, so they are fetched with
+// scalar loads into SGPRs; every gathered X row segment X[j, c0 .. c0+64*VEC) is
+// one fully coalesced vector load; each lane keeps VEC fp32 accumulators that
+// start at bias[i] and receive one fused multiply-add per stored nonzero in
+// ascending slot order -- the rounding sequence of the reference's inner loop
+// (src/ellpack_matmul.cpp:51-66) -- followed by the fused epilogue.
+//
+// Workgroups are numbered so that each of the 8 XCDs (workgroup id modulo 8)
+// works on as few column tiles as possible: an XCD's L2 then has to hold only
+// its own tiles' slice of X.
+#include "so_internal.h"
+
+namespace {
+
+constexpr int kWavesPerGroup = 4;
+constexpr int kUnroll = 8;
+
+template <int VEC> struct VecT;
+template <> struct VecT<1> { using type = float; };
+template <> struct VecT<2> { using type = float2; };
+template <> struct VecT<4> { using type = float4; };
+
+template <int VEC>
+__device__ __forceinline__ void load_vec(const float *p, float (&v)[VEC])
+{
+    using T = typename VecT<VEC>::type;
+    const T t = *reinterpret_cast<const T *>(p);
+    if constexpr (VEC == 1) { v[0] = t; }
+    if constexpr (VEC == 2) { v[0] = t.x; v[1] = t.y; }
+    if constexpr (VEC == 4) { v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+}
+
+template <int VEC>
+__device__ __forceinline__ void store_vec(float *p, const float (&v)[VEC])
+{
+    using T = typename VecT<VEC>::type;
+    T t;
+    if constexpr (VEC == 1) { t = v[0]; }
+    if constexpr (VEC == 2) { t.x = v[0]; t.y = v[1]; }
+    if constexpr (VEC == 4) { t.x = v[0]; t.y = v[1]; t.z = v[2]; t.w = v[3]; }
+    *reinterpret_cast<T *>(p) = t;
+}
+
+struct TileMap {
+    uint32_t ntiles;      // column tiles
+    uint32_t nrowgroups;  // groups of kWavesPerGroup rows
+    uint32_t mode;        // 0 plain, 1: ntiles divides 8, 2: 8 divides ntiles
+};
+
+// Workgroup id -> (column tile, row group).  XCD = id % 8.
+__device__ __forceinline__ bool map_tile(const TileMap tm, uint32_t wg, uint32_t &tile, uint32_t &rg)
+{
+    const uint32_t xcd = wg & 7u, q = wg >> 3;
+    if (tm.mode == 1) {
+        const uint32_t per = 8u / tm.ntiles;  // XCDs sharing one tile
+        tile = xcd % tm.ntiles;
+        rg = xcd / tm.ntiles + per * q;
+    } else if (tm.mode == 2) {
+        const uint32_t per = tm.ntiles >> 3;  // tiles per XCD
+        tile = xcd + 8u * (q % per);
+        rg = q / per;
+    } else {
+        tile = wg % tm.ntiles;
+        rg = wg / tm.ntiles;
+    }
+    return rg < tm.nrowgroups;
+}
+
+// FULL: every column tile is complete (C % (64*VEC) == 0), no lane predicate.
+template <int VEC, int ACT, bool FULL>
+__global__ __launch_bounds__(kWavesPerGroup * 64)
+void ellpack_matmul_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
+                           const uint32_t *__restrict__ nnz, uint32_t m, uint32_t r,
+                           const float *__restrict__ X, uint32_t C,
+                           const float *__restrict__ bias, float *__restrict__ Y, TileMap tm)
+{
+    uint32_t tile, rg;
+    if (!map_tile(tm, blockIdx.x, tile, rg)) return;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t row = __builtin_amdgcn_readfirstlane(rg * kWavesPerGroup + (threadIdx.x >> 6));
+    if (row >= m) return;
+
+    const uint32_t col = tile * (64u * VEC) + lane * VEC;
+    // A partial tile only happens with VEC == 1 (the host picks VEC so that C % VEC == 0).
+    const bool live = FULL || col < C;
+    const uint32_t cnt = nnz[row];
+    const float *__restrict__ wrow = Wd + (size_t)row * r;
+    const uint32_t *__restrict__ irow = idx + (size_t)row * r;
+    const float *__restrict__ xcol = X + (live ? col : 0u);
+
+    float acc[VEC];
+    const float b = bias ? bias[row] : 0.0f;
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = b;
+
+    uint32_t j = 0;
+    for (; j + kUnroll <= cnt; j += kUnroll) {
+        float w[kUnroll];
+        float x[kUnroll][VEC];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            w[u] = wrow[j + u];
+            load_vec<VEC>(xcol + (size_t)irow[j + u] * C, x[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(w[u], x[u][v], acc[v]);
+    }
+    for (; j < cnt; ++j) {
+        const float w = wrow[j];
+        float x[VEC];
+        load_vec<VEC>(xcol + (size_t)irow[j] * C, x);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(w, x[v], acc[v]);
+    }
+
+    if (live) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = so_epilogue<ACT>(acc[v]);
+        store_vec<VEC>(Y + (size_t)row * C + col, acc);
+    }
+}
+
+template <int VEC, int ACT>
+void launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, const float *dBias, float *dY)
+{
+    TileMap tm;
+    tm.ntiles = so_ceil_div(C, 64u * VEC);
+    tm.nrowgroups = so_ceil_div(E->m, kWavesPerGroup);
+    tm.mode = (tm.ntiles <= 8 && 8 % tm.ntiles == 0) ? 1 : (tm.ntiles % 8 == 0 ? 2 : 0);
+    uint32_t blocks;
+    if (tm.mode == 1) blocks = so_ceil_div(tm.nrowgroups, 8u / tm.ntiles) * 8u;
+    else blocks = tm.ntiles * tm.nrowgroups;
+    const bool full = C % (64u * VEC) == 0;
+    auto k = full ? ellpack_matmul_kernel<VEC, ACT, true> : ellpack_matmul_kernel<VEC, ACT, false>;
+    k<<<blocks, kWavesPerGroup * 64, 0, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->r,
+                                                       dX, C, dBias, dY, tm);
+}
+
+template <int VEC>
+void launch_act(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, const float *dBias,
+                float *dY, int act)
+{
+    switch (act) {
+    case SO_ACT_RELU:    launch<VEC, SO_ACT_RELU>(ctx, E, dX, C, dBias, dY); break;
+    case SO_ACT_SIGMOID: launch<VEC, SO_ACT_SIGMOID>(ctx, E, dX, C, dBias, dY); break;
+    case SO_ACT_TANH:    launch<VEC, SO_ACT_TANH>(ctx, E, dX, C, dBias, dY); break;
+    default:             launch<VEC, SO_ACT_NONE>(ctx, E, dX, C, dBias, dY); break;
+    }
+}
+
+} // namespace
+
+extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
+                               const float *dBias, float *dY, int act)
+{
+    SO_REQUIRE(ctx && E, "so_matmul: null argument");
+    SO_REQUIRE(act >= SO_ACT_NONE && act <= SO_ACT_TANH, "so_matmul: unknown activation %d", act);
+    if (E->m == 0 || C == 0) return SO_OK;  // empty output: nothing to launch
+    SO_REQUIRE(dY != nullptr, "so_matmul: Y is null");
+    SO_REQUIRE(dX != nullptr || E->total_nnz == 0, "so_matmul: X is null");
+
+    // Columns per lane: as wide as alignment allows while every tile stays whole.
+    const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY;
+    int vec = 1;
+    if (C % 256 == 0 && (align & 15) == 0) vec = 4;
+    else if (C % 128 == 0 && (align & 7) == 0) vec = 2;
+    if (vec == 4) launch_act<4>(ctx, E, dX, C, dBias, dY, act);
+    else if (vec == 2) launch_act<2>(ctx, E, dX, C, dBias, dY, act);
+    else launch_act<1>(ctx, E, dX, C, dBias, dY, act);
+    SO_LAUNCH_CHECK();
+    return SO_OK;
+}

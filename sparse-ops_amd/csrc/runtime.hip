@@ -1,0 +1,385 @@
+// Context, memory, timing, launch graphs and the device-resident ELLPACK layouts.
+#include "so_internal.h"
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstring>
+#include <new>
+
+static thread_local std::string g_last_error;
+
+void so_set_error(const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+}
+
+extern "C" const char *so_last_error(void) { return g_last_error.c_str(); }
+
+extern "C" so_status so_device_count(int *n)
+{
+    SO_REQUIRE(n != nullptr, "so_device_count: n is null");
+    *n = 0;
+    int c = 0;
+    hipError_t e = hipGetDeviceCount(&c);
+    if (e != hipSuccess || c <= 0) {
+        (void)hipGetLastError();
+        so_set_error("no HIP device available (%s)", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+        return SO_ERR_NO_DEVICE;
+    }
+    *n = c;
+    return SO_OK;
+}
+
+extern "C" so_status so_init(int device, so_ctx **out)
+{
+    SO_REQUIRE(out != nullptr, "so_init: out is null");
+    *out = nullptr;
+    int c = 0;
+    so_status s = so_device_count(&c);
+    if (s != SO_OK) return s;
+    SO_REQUIRE(device >= 0 && device < c, "so_init: device %d out of range (have %d)", device, c);
+    SO_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    SO_HIP(hipGetDeviceProperties(&prop, device));
+    so_ctx *ctx = new (std::nothrow) so_ctx();
+    if (!ctx) { so_set_error("so_init: host allocation failed"); return SO_ERR_OOM; }
+    ctx->device = device;
+    ctx->compute_units = prop.multiProcessorCount;
+    ctx->max_lds_bytes = (int)prop.sharedMemPerBlock;
+    ctx->name = prop.gcnArchName;
+    hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreate(&ctx->ev0);
+    if (e == hipSuccess) e = hipEventCreate(&ctx->ev1);
+    if (e != hipSuccess) {
+        so_set_error("so_init: stream/event creation failed: %s", hipGetErrorString(e));
+        so_destroy(ctx);
+        return SO_ERR_HIP;
+    }
+    *out = ctx;
+    return SO_OK;
+}
+
+extern "C" so_status so_destroy(so_ctx *ctx)
+{
+    if (!ctx) return SO_OK;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) { (void)hipStreamSynchronize(ctx->stream); (void)hipStreamDestroy(ctx->stream); }
+    if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
+    if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+    delete ctx;
+    return SO_OK;
+}
+
+extern "C" so_status so_device_info(so_ctx *ctx, char *name, size_t name_len, int *compute_units)
+{
+    SO_REQUIRE(ctx != nullptr, "so_device_info: ctx is null");
+    if (name && name_len) {
+        std::strncpy(name, ctx->name.c_str(), name_len - 1);
+        name[name_len - 1] = '\0';
+    }
+    if (compute_units) *compute_units = ctx->compute_units;
+    return SO_OK;
+}
+
+extern "C" so_status so_malloc(so_ctx *ctx, size_t bytes, void **dptr)
+{
+    SO_REQUIRE(ctx && dptr, "so_malloc: null argument");
+    SO_REQUIRE(!ctx->capturing, "so_malloc: not allowed while a graph is being recorded");
+    *dptr = nullptr;
+    if (bytes == 0) bytes = 4;  // a valid, distinct pointer even for empty tensors
+    SO_HIP(hipSetDevice(ctx->device));
+    SO_HIP(hipMalloc(dptr, bytes));
+    return SO_OK;
+}
+
+extern "C" so_status so_free(so_ctx *ctx, void *dptr)
+{
+    SO_REQUIRE(ctx != nullptr, "so_free: ctx is null");
+    if (!dptr) return SO_OK;
+    SO_REQUIRE(!ctx->capturing, "so_free: not allowed while a graph is being recorded");
+    SO_HIP(hipStreamSynchronize(ctx->stream));
+    SO_HIP(hipFree(dptr));
+    return SO_OK;
+}
+
+extern "C" so_status so_h2d(so_ctx *ctx, void *dst, const void *src, size_t bytes)
+{
+    SO_REQUIRE(ctx != nullptr, "so_h2d: ctx is null");
+    if (bytes == 0) return SO_OK;
+    SO_REQUIRE(dst && src, "so_h2d: null pointer");
+    SO_REQUIRE(!ctx->capturing, "so_h2d: not allowed while a graph is being recorded");
+    SO_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    SO_HIP(hipStreamSynchronize(ctx->stream));
+    return SO_OK;
+}
+
+extern "C" so_status so_d2h(so_ctx *ctx, void *dst, const void *src, size_t bytes)
+{
+    SO_REQUIRE(ctx != nullptr, "so_d2h: ctx is null");
+    if (bytes == 0) return SO_OK;
+    SO_REQUIRE(dst && src, "so_d2h: null pointer");
+    SO_REQUIRE(!ctx->capturing, "so_d2h: not allowed while a graph is being recorded");
+    SO_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    SO_HIP(hipStreamSynchronize(ctx->stream));
+    return SO_OK;
+}
+
+extern "C" so_status so_d2d(so_ctx *ctx, void *dst, const void *src, size_t bytes)
+{
+    SO_REQUIRE(ctx != nullptr, "so_d2d: ctx is null");
+    if (bytes == 0) return SO_OK;
+    SO_REQUIRE(dst && src, "so_d2d: null pointer");
+    SO_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return SO_OK;
+}
+
+__global__ void so_fill_zero_kernel(uint32_t *p, size_t words)
+{
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < words; i += stride) p[i] = 0u;
+}
+
+extern "C" so_status so_fill_zero(so_ctx *ctx, void *dptr, size_t bytes)
+{
+    SO_REQUIRE(ctx != nullptr, "so_fill_zero: ctx is null");
+    if (bytes == 0) return SO_OK;
+    SO_REQUIRE(dptr != nullptr && bytes % 4 == 0 && ((uintptr_t)dptr & 3) == 0,
+               "so_fill_zero: pointer and size must be 4-byte multiples");
+    const size_t words = bytes / 4;
+    const uint32_t blocks = (uint32_t)std::min<size_t>((words + 255) / 256, 4096);
+    so_fill_zero_kernel<<<blocks, 256, 0, ctx->stream>>>((uint32_t *)dptr, words);
+    SO_LAUNCH_CHECK();
+    return SO_OK;
+}
+
+extern "C" so_status so_sync(so_ctx *ctx)
+{
+    SO_REQUIRE(ctx != nullptr, "so_sync: ctx is null");
+    SO_REQUIRE(!ctx->capturing, "so_sync: not allowed while a graph is being recorded");
+    SO_HIP(hipStreamSynchronize(ctx->stream));
+    return SO_OK;
+}
+
+extern "C" so_status so_timer_begin(so_ctx *ctx)
+{
+    SO_REQUIRE(ctx != nullptr, "so_timer_begin: ctx is null");
+    SO_REQUIRE(!ctx->capturing, "so_timer_begin: not allowed while a graph is being recorded");
+    SO_HIP(hipEventRecord(ctx->ev0, ctx->stream));
+    return SO_OK;
+}
+
+extern "C" so_status so_timer_end(so_ctx *ctx, float *ms)
+{
+    SO_REQUIRE(ctx && ms, "so_timer_end: null argument");
+    SO_REQUIRE(!ctx->capturing, "so_timer_end: not allowed while a graph is being recorded");
+    SO_HIP(hipEventRecord(ctx->ev1, ctx->stream));
+    SO_HIP(hipEventSynchronize(ctx->ev1));
+    SO_HIP(hipEventElapsedTime(ms, ctx->ev0, ctx->ev1));
+    return SO_OK;
+}
+
+// ---------------------------------------------------------------- launch graphs
+
+extern "C" so_status so_graph_begin(so_ctx *ctx)
+{
+    SO_REQUIRE(ctx != nullptr, "so_graph_begin: ctx is null");
+    SO_REQUIRE(!ctx->capturing, "so_graph_begin: already recording");
+    SO_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return SO_OK;
+}
+
+extern "C" so_status so_graph_end(so_ctx *ctx, so_graph **out)
+{
+    SO_REQUIRE(ctx && out, "so_graph_end: null argument");
+    SO_REQUIRE(ctx->capturing, "so_graph_end: not recording");
+    *out = nullptr;
+    ctx->capturing = false;
+    hipGraph_t graph = nullptr;
+    SO_HIP(hipStreamEndCapture(ctx->stream, &graph));
+    so_graph *g = new (std::nothrow) so_graph();
+    if (!g) { (void)hipGraphDestroy(graph); so_set_error("so_graph_end: host allocation failed"); return SO_ERR_OOM; }
+    g->graph = graph;
+    hipError_t e = hipGraphInstantiate(&g->exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        so_set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
+        (void)hipGraphDestroy(graph);
+        delete g;
+        return SO_ERR_HIP;
+    }
+    *out = g;
+    return SO_OK;
+}
+
+extern "C" so_status so_graph_launch(so_ctx *ctx, so_graph *g)
+{
+    SO_REQUIRE(ctx && g && g->exec, "so_graph_launch: null argument");
+    SO_REQUIRE(!ctx->capturing, "so_graph_launch: not allowed while recording");
+    SO_HIP(hipGraphLaunch(g->exec, ctx->stream));
+    return SO_OK;
+}
+
+extern "C" so_status so_graph_free(so_ctx *ctx, so_graph *g)
+{
+    if (!g) return SO_OK;
+    if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    delete g;
+    return SO_OK;
+}
+
+// ------------------------------------------------------------ ELLPACK on device
+
+static void free_ellpack_arrays(so_ellpack *E)
+{
+    if (E->d_Wd) (void)hipFree(E->d_Wd);
+    if (E->d_idx) (void)hipFree(E->d_idx);
+    if (E->d_nnz) (void)hipFree(E->d_nnz);
+    if (E->d_WdT) (void)hipFree(E->d_WdT);
+    if (E->d_idxT) (void)hipFree(E->d_idxT);
+    for (auto &b : E->bins)
+        if (b.d_rows) (void)hipFree(b.d_rows);
+}
+
+// Device copy of a host array with 16 zeroed bytes after the last element, so a
+// kernel may read whole aligned 16-byte groups that straddle the end.
+template <typename T>
+static so_status upload_array(so_ctx *ctx, const T *host, size_t count, T **dev)
+{
+    void *p = nullptr;
+    so_status s = so_malloc(ctx, count * sizeof(T) + 16, &p);
+    if (s != SO_OK) return s;
+    *dev = (T *)p;
+    SO_HIP(hipMemsetAsync((char *)p + count * sizeof(T), 0, 16, ctx->stream));
+    return so_h2d(ctx, p, host, count * sizeof(T));
+}
+
+extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint32_t *idx,
+                                       const uint32_t *nnz, uint32_t m, uint32_t n, uint32_t r,
+                                       int layouts, so_ellpack **out)
+{
+    SO_REQUIRE(ctx && out, "so_ellpack_upload: null argument");
+    *out = nullptr;
+    const size_t slots = (size_t)m * r;
+    SO_REQUIRE(m == 0 || nnz != nullptr, "so_ellpack_upload: nnz is null");
+    SO_REQUIRE(slots == 0 || (Wd && idx), "so_ellpack_upload: Wd/idx is null");
+    SO_REQUIRE((layouts & ~(SO_LAYOUT_ROW | SO_LAYOUT_SLOT | SO_LAYOUT_BINS)) == 0,
+               "so_ellpack_upload: unknown layout bits 0x%x", layouts);
+
+    // Validate on the host before anything reaches a kernel: every stored slot must
+    // name a column inside X, every count must fit the row.
+    uint64_t total = 0;
+    uint32_t max_nnz = 0;
+    for (uint32_t i = 0; i < m; ++i) {
+        const uint32_t c = nnz[i];
+        if (c > r) {
+            so_set_error("so_ellpack_upload: nnz[%u] = %u exceeds r = %u", i, c, r);
+            return SO_ERR_BOUNDS;
+        }
+        const uint32_t *row = idx + (size_t)i * r;
+        for (uint32_t k = 0; k < c; ++k)
+            if (row[k] >= n) {
+                so_set_error("so_ellpack_upload: idx[%u,%u] = %u is not below n = %u", i, k, row[k], n);
+                return SO_ERR_BOUNDS;
+            }
+        total += c;
+        max_nnz = std::max(max_nnz, c);
+    }
+
+    so_ellpack *E = new (std::nothrow) so_ellpack();
+    if (!E) { so_set_error("so_ellpack_upload: host allocation failed"); return SO_ERR_OOM; }
+    E->m = m; E->n = n; E->r = r;
+    E->total_nnz = total;
+    E->max_nnz = max_nnz;
+    E->layouts = layouts | SO_LAYOUT_ROW;
+
+    so_status s = upload_array(ctx, Wd, slots, &E->d_Wd);
+    if (s == SO_OK) s = upload_array(ctx, idx, slots, &E->d_idx);
+    if (s == SO_OK) s = upload_array(ctx, nnz, (size_t)m, &E->d_nnz);
+
+    if (s == SO_OK && (layouts & SO_LAYOUT_SLOT)) {
+        std::vector<float> WdT(slots);
+        std::vector<uint32_t> idxT(slots);
+        for (uint32_t i = 0; i < m; ++i)
+            for (uint32_t k = 0; k < r; ++k) {
+                WdT[(size_t)k * m + i] = Wd[(size_t)i * r + k];
+                idxT[(size_t)k * m + i] = idx[(size_t)i * r + k];
+            }
+        s = upload_array(ctx, WdT.data(), slots, &E->d_WdT);
+        if (s == SO_OK) s = upload_array(ctx, idxT.data(), slots, &E->d_idxT);
+    }
+
+    if (s == SO_OK && (layouts & SO_LAYOUT_BINS)) {
+        // Length classes: <= 16 nonzeros -> 4 lanes per row, <= 128 -> 16 lanes,
+        // longer -> a whole wave.  Long rows first inside a class, so the last
+        // waves to start are the short ones.
+        static const uint32_t group[3] = {4, 16, 64};
+        static const uint32_t limit[3] = {16, 128, 0xffffffffu};
+        std::vector<uint32_t> rows[3];
+        for (uint32_t i = 0; i < m; ++i) {
+            int b = 0;
+            while (nnz[i] > limit[b]) ++b;
+            rows[b].push_back(i);
+        }
+        for (int b = 0; b < 3 && s == SO_OK; ++b) {
+            std::stable_sort(rows[b].begin(), rows[b].end(),
+                             [&](uint32_t a, uint32_t c) { return nnz[a] > nnz[c]; });
+            E->bins[b].group = group[b];
+            E->bins[b].count = (uint32_t)rows[b].size();
+            if (!rows[b].empty()) s = upload_array(ctx, rows[b].data(), rows[b].size(), &E->bins[b].d_rows);
+        }
+    }
+
+    if (s != SO_OK) {
+        free_ellpack_arrays(E);
+        delete E;
+        return s;
+    }
+    *out = E;
+    return SO_OK;
+}
+
+extern "C" so_status so_ellpack_free(so_ctx *ctx, so_ellpack *E)
+{
+    if (!E) return SO_OK;
+    if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    free_ellpack_arrays(E);
+    delete E;
+    return SO_OK;
+}
+
+extern "C" so_status so_ellpack_dims(const so_ellpack *E, uint32_t *m, uint32_t *n, uint32_t *r,
+                                     uint64_t *total_nnz, int *layouts)
+{
+    SO_REQUIRE(E != nullptr, "so_ellpack_dims: E is null");
+    if (m) *m = E->m;
+    if (n) *n = E->n;
+    if (r) *r = E->r;
+    if (total_nnz) *total_nnz = E->total_nnz;
+    if (layouts) *layouts = E->layouts;
+    return SO_OK;
+}
+
+extern "C" so_status so_ellpack_download(so_ctx *ctx, const so_ellpack *E, int layout,
+                                         float *Wd, uint32_t *idx, uint32_t *nnz)
+{
+    SO_REQUIRE(ctx && E, "so_ellpack_download: null argument");
+    SO_REQUIRE(layout == SO_LAYOUT_ROW || layout == SO_LAYOUT_SLOT,
+               "so_ellpack_download: layout must be ROW or SLOT");
+    SO_REQUIRE((E->layouts & layout) != 0, "so_ellpack_download: layout %d was not uploaded", layout);
+    const size_t slots = (size_t)E->m * E->r;
+    const float *w = layout == SO_LAYOUT_ROW ? E->d_Wd : E->d_WdT;
+    const uint32_t *ix = layout == SO_LAYOUT_ROW ? E->d_idx : E->d_idxT;
+    so_status s = SO_OK;
+    if (Wd && slots) s = so_d2h(ctx, Wd, w, slots * sizeof(float));
+    if (s == SO_OK && idx && slots) s = so_d2h(ctx, idx, ix, slots * sizeof(uint32_t));
+    if (s == SO_OK && nnz && E->m) s = so_d2h(ctx, nnz, E->d_nnz, (size_t)E->m * sizeof(uint32_t));
+    return s;
+}

@@ -1,0 +1,88 @@
+// Internal definitions shared by the HIP translation units of libsparseops_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "sparseops_hip.h"
+
+struct so_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    int compute_units = 0;
+    int max_lds_bytes = 0;   // largest LDS allocation one workgroup may ask for
+    bool capturing = false;
+    std::string name;
+};
+
+// Rows of one length class for the binned matvec: `group` lanes cooperate on a row.
+struct so_bin {
+    uint32_t group = 0;      // 4, 16 or 64 lanes per row
+    uint32_t count = 0;      // rows in this class
+    uint32_t *d_rows = nullptr;
+};
+
+struct so_ellpack {
+    uint32_t m = 0, n = 0, r = 0;
+    uint64_t total_nnz = 0;
+    uint32_t max_nnz = 0;
+    int layouts = 0;
+    float *d_Wd = nullptr;       // [m*r] row-major
+    uint32_t *d_idx = nullptr;   // [m*r]
+    uint32_t *d_nnz = nullptr;   // [m]
+    float *d_WdT = nullptr;      // [r*m] slot-major (SO_LAYOUT_SLOT)
+    uint32_t *d_idxT = nullptr;
+    so_bin bins[3];              // SO_LAYOUT_BINS
+};
+
+struct so_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+void so_set_error(const char *fmt, ...);
+
+#define SO_HIP(call)                                                              \
+    do {                                                                          \
+        hipError_t e_ = (call);                                                   \
+        if (e_ != hipSuccess) {                                                   \
+            so_set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_),   \
+                         __FILE__, __LINE__);                                     \
+            return e_ == hipErrorOutOfMemory ? SO_ERR_OOM : SO_ERR_HIP;           \
+        }                                                                         \
+    } while (0)
+
+#define SO_REQUIRE(cond, ...)                                                     \
+    do {                                                                          \
+        if (!(cond)) {                                                            \
+            so_set_error(__VA_ARGS__);                                            \
+            return SO_ERR_INVALID;                                                \
+        }                                                                         \
+    } while (0)
+
+// Launch check that is valid both eagerly and while a graph is being recorded.
+#define SO_LAUNCH_CHECK()                                                         \
+    do {                                                                          \
+        hipError_t e_ = hipGetLastError();                                        \
+        if (e_ != hipSuccess) {                                                   \
+            so_set_error("kernel launch failed: %s (%s:%d)", hipGetErrorString(e_), \
+                         __FILE__, __LINE__);                                     \
+            return SO_ERR_HIP;                                                    \
+        }                                                                         \
+    } while (0)
+
+static inline uint32_t so_ceil_div(uint64_t a, uint64_t b) { return (uint32_t)((a + b - 1) / b); }
+
+// Epilogue shared by the matmul and conv kernels.  expf/tanhf are the accurate
+// OCML routines (no fast-math), matching 1.0f/(1.0f+expf(-v)) and tanhf(v).
+template <int ACT>
+__device__ __forceinline__ float so_epilogue(float v)
+{
+    if (ACT == SO_ACT_RELU) return v > 0.0f ? v : 0.0f;
+    if (ACT == SO_ACT_SIGMOID) return 1.0f / (1.0f + expf(-v));
+    if (ACT == SO_ACT_TANH) return tanhf(v);
+    return v;
+}

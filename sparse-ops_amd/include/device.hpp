@@ -1,0 +1,61 @@
+// C++ convenience layer over the C ABI (include/sparseops_hip.h): one process-wide
+// context, RAII device buffers, and the translation of status codes into the
+// exception types the reference's callers see (std::runtime_error).
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <mutex>
+#include <stdexcept>
+#include <string>
+
+#include "sparseops_hip.h"
+
+struct Ellpack;
+
+namespace sparseops {
+
+/// Throws std::runtime_error("<what>: <so_last_error()>") unless st == SO_OK
+/// (std::bad_alloc for SO_ERR_OOM).
+void check(so_status st, const char *what);
+
+/// The process-wide context on device 0, created on first use.
+/// Throws std::runtime_error if no HIP device is usable.
+so_ctx *context();
+/// Serialises host-pointer calls that share the staging buffers.
+std::mutex &context_mutex();
+
+class DeviceBuffer {
+public:
+    DeviceBuffer() = default;
+    explicit DeviceBuffer(std::size_t bytes) { reserve(bytes); }
+    ~DeviceBuffer();
+    DeviceBuffer(const DeviceBuffer &) = delete;
+    DeviceBuffer &operator=(const DeviceBuffer &) = delete;
+    DeviceBuffer(DeviceBuffer &&o) noexcept : ptr_(o.ptr_), bytes_(o.bytes_) { o.ptr_ = nullptr; o.bytes_ = 0; }
+    DeviceBuffer &operator=(DeviceBuffer &&o) noexcept;
+
+    /// Grow-only: reallocates (contents lost) when `bytes` exceeds the capacity.
+    void reserve(std::size_t bytes);
+    void release();
+    float *f32() const { return static_cast<float *>(ptr_); }
+    void *get() const { return ptr_; }
+    std::size_t bytes() const { return bytes_; }
+
+private:
+    void *ptr_ = nullptr;
+    std::size_t bytes_ = 0;
+};
+
+/// Device copy of an Ellpack, owned through Ellpack::device.
+struct EllpackMirror {
+    so_ellpack *handle = nullptr;
+    int layouts = 0;
+    ~EllpackMirror();
+};
+
+/// Upload E once (or again if `layouts` asks for more than is resident) and
+/// return the device handle.
+const so_ellpack *mirror(const Ellpack &E, int layouts);
+
+} // namespace sparseops

@@ -1,0 +1,80 @@
+// Host-pointer entry points with the reference's signatures, executed on the GPU:
+// device copy of E (cached) + upload of X/bias + HIP kernel + download of Y.
+#include "ellpack_matmul.hpp"
+#include "ellpack_matvec.hpp"
+
+#include "device.hpp"
+
+namespace {
+
+// Grow-only staging buffers shared by all host-pointer calls of the process.
+struct Staging {
+    sparseops::DeviceBuffer x, y, bias;
+};
+Staging &staging()
+{
+    static Staging *s = new Staging();  // intentionally leaked: freed with the process
+    return *s;
+}
+
+void matmul_host(const Ellpack &E, const float *X, uint32_t C, const float *bias, float *Y, int act)
+{
+    using namespace sparseops;
+    so_ctx *ctx = context();
+    std::lock_guard<std::mutex> lock(context_mutex());
+    if (E.m == 0 || C == 0) return;
+    const so_ellpack *dE = mirror(E, SO_LAYOUT_ROW);
+    Staging &st = staging();
+    const std::size_t xbytes = std::size_t(E.n) * C * sizeof(float);
+    const std::size_t ybytes = std::size_t(E.m) * C * sizeof(float);
+    st.x.reserve(xbytes);
+    st.y.reserve(ybytes);
+    check(so_h2d(ctx, st.x.get(), X, xbytes), "so_h2d(X)");
+    const float *dBias = nullptr;
+    if (bias) {
+        st.bias.reserve(std::size_t(E.m) * sizeof(float));
+        check(so_h2d(ctx, st.bias.get(), bias, std::size_t(E.m) * sizeof(float)), "so_h2d(bias)");
+        dBias = st.bias.f32();
+    }
+    check(so_matmul(ctx, dE, st.x.f32(), C, dBias, st.y.f32(), act), "so_matmul");
+    check(so_d2h(ctx, Y, st.y.get(), ybytes), "so_d2h(Y)");
+}
+
+} // namespace
+
+template <bool USE_MASK, bool FUSE_RELU>
+void ellpack_matmul_fused(const Ellpack &E, const float *X, uint32_t C, const float *bias, float *Y)
+{
+    matmul_host(E, X, C, bias, Y, FUSE_RELU ? SO_ACT_RELU : SO_ACT_NONE);
+}
+
+template void ellpack_matmul_fused<false, false>(const Ellpack &, const float *, uint32_t, const float *, float *);
+template void ellpack_matmul_fused<false, true>(const Ellpack &, const float *, uint32_t, const float *, float *);
+template void ellpack_matmul_fused<true, false>(const Ellpack &, const float *, uint32_t, const float *, float *);
+template void ellpack_matmul_fused<true, true>(const Ellpack &, const float *, uint32_t, const float *, float *);
+
+void ellpack_matvec(const Ellpack &E, const float *x, const float *bias, float *y)
+{
+    using namespace sparseops;
+    so_ctx *ctx = context();
+    std::lock_guard<std::mutex> lock(context_mutex());
+    if (E.m == 0) return;
+    // Skewed row lengths (widest row far above the mean): keep length classes so
+    // that padding is never streamed and short rows do not occupy whole waves.
+    uint64_t total = 0;
+    for (uint32_t c : E.nnz) total += c;
+    const bool skewed = uint64_t(E.r) * E.m > 2 * total + E.m;
+    const so_ellpack *dE = mirror(E, skewed ? (SO_LAYOUT_ROW | SO_LAYOUT_BINS) : SO_LAYOUT_ROW);
+    Staging &st = staging();
+    st.x.reserve(std::size_t(E.n) * sizeof(float));
+    st.y.reserve(std::size_t(E.m) * sizeof(float));
+    check(so_h2d(ctx, st.x.get(), x, std::size_t(E.n) * sizeof(float)), "so_h2d(x)");
+    const float *dBias = nullptr;
+    if (bias) {
+        st.bias.reserve(std::size_t(E.m) * sizeof(float));
+        check(so_h2d(ctx, st.bias.get(), bias, std::size_t(E.m) * sizeof(float)), "so_h2d(bias)");
+        dBias = st.bias.f32();
+    }
+    check(so_matvec(ctx, dE, st.x.f32(), dBias, st.y.f32(), skewed ? SO_LAYOUT_BINS : SO_LAYOUT_ROW), "so_matvec");
+    check(so_d2h(ctx, y, st.y.get(), std::size_t(E.m) * sizeof(float)), "so_d2h(y)");
+}

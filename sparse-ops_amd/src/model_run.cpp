@@ -1,0 +1,117 @@
+// SparseOnnxModel: buffer sizing and execution.  The reference walks the layers
+// with a name->buffer map and allocates every output per call
+// (src/model_run.cpp:3-140, src/layers/*.cpp); here every tensor has a fixed slot
+// in one HBM arena, the chain is recorded once into a launch graph, and a call
+// with an unchanged batch size allocates nothing.
+#include "sparse_onnx.hpp"
+
+#include <stdexcept>
+
+#include "model_impl.hpp"
+
+using namespace sparseops;
+
+void SparseOnnxModel::resize_buffers(uint32_t batch)
+{
+    Impl &M = *impl_;
+    if (batch == 0) throw std::runtime_error("resize_buffers: batch must be positive");
+    so_ctx *ctx = context();
+    std::lock_guard<std::mutex> lock(context_mutex());
+    if (M.graph) { so_graph_free(ctx, M.graph); M.graph = nullptr; }
+    // Slot offsets for this batch, 256-byte aligned.
+    std::size_t total = 0;
+    for (Slot &s : M.slots) {
+        s.offset = total;
+        total += (s.features * batch + 63) / 64 * 64;
+    }
+    M.arena.reserve(total * sizeof(float));
+    M.stage_in.reserve(M.in_features * batch * sizeof(float));
+    M.stage_out.reserve(M.out_features * batch * sizeof(float));
+    M.batch = batch;
+    if (M.use_graph && !M.layers.empty()) {
+        check(so_graph_begin(ctx), "so_graph_begin");
+        try {
+            M.enqueue_layers(nullptr, nullptr);
+        } catch (...) {
+            so_graph *g = nullptr;
+            so_graph_end(ctx, &g);
+            so_graph_free(ctx, g);
+            throw;
+        }
+        check(so_graph_end(ctx, &M.graph), "so_graph_end");
+    }
+}
+
+void SparseOnnxModel::Impl::enqueue_layers(const float *in, float *out) const
+{
+    so_ctx *ctx = context();
+    const uint32_t B = batch;
+    auto src = [&](int s) -> const float * { return (in && s == input_slot) ? in : slot_ptr(s); };
+    auto dst = [&](int s) -> float * { return (out && s == output_slot) ? out : slot_ptr(s); };
+    for (const LayerPlan &L : layers) {
+        const float *bias = L.has_bias ? bias_pool.f32() + L.bias_offset : nullptr;
+        switch (L.op) {
+        case Op::MatMul:
+            check(so_matmul(ctx, L.dE, src(L.in0), B, bias, dst(L.out), L.act), "so_matmul");
+            break;
+        case Op::Conv:
+            check(so_conv2d(ctx, L.conv, src(L.in0), B, bias, dst(L.out), L.act), "so_conv2d");
+            break;
+        case Op::Act:
+            check(so_act(ctx, L.act, src(L.in0), L.out_features * B, dst(L.out)), "so_act");
+            break;
+        case Op::Add:
+            check(so_add(ctx, src(L.in0), src(L.in1), L.out_features * B, dst(L.out)), "so_add");
+            break;
+        case Op::MaxPool:
+            check(so_maxpool(ctx, &L.pg, src(L.in0), B, dst(L.out)), "so_maxpool");
+            break;
+        case Op::GlobalAveragePool:
+            check(so_gap(ctx, L.pg.C, L.pg.H, L.pg.W, src(L.in0), B, dst(L.out)), "so_gap");
+            break;
+        }
+    }
+}
+
+void SparseOnnxModel::Impl::launch_chain() const
+{
+    if (graph) check(so_graph_launch(context(), graph), "so_graph_launch");
+    else enqueue_layers(nullptr, nullptr);
+}
+
+void SparseOnnxModel::run(const float *input, uint32_t B, float *output) const
+{
+    Impl &M = *impl_;
+    if (B != M.batch) const_cast<SparseOnnxModel *>(this)->resize_buffers(B);
+    so_ctx *ctx = context();
+    std::lock_guard<std::mutex> lock(context_mutex());
+    check(so_h2d(ctx, M.slot_ptr(M.input_slot), input, M.in_features * B * sizeof(float)), "so_h2d(input)");
+    M.launch_chain();
+    check(so_d2h(ctx, output, M.slot_ptr(M.output_slot), M.out_features * B * sizeof(float)), "so_d2h(output)");
+}
+
+void SparseOnnxModel::run_batch_major(const float *input, uint32_t B, float *output) const
+{
+    Impl &M = *impl_;
+    if (B != M.batch) const_cast<SparseOnnxModel *>(this)->resize_buffers(B);
+    so_ctx *ctx = context();
+    std::lock_guard<std::mutex> lock(context_mutex());
+    check(so_h2d(ctx, M.stage_in.get(), input, M.in_features * B * sizeof(float)), "so_h2d(input)");
+    check(so_transpose(ctx, M.stage_in.f32(), B, uint32_t(M.in_features), M.slot_ptr(M.input_slot)), "so_transpose(input)");
+    M.launch_chain();
+    check(so_transpose(ctx, M.slot_ptr(M.output_slot), uint32_t(M.out_features), B, M.stage_out.f32()), "so_transpose(output)");
+    check(so_d2h(ctx, output, M.stage_out.get(), M.out_features * B * sizeof(float)), "so_d2h(output)");
+}
+
+void SparseOnnxModel::run_device(const float *dInput, uint32_t B, float *dOutput) const
+{
+    Impl &M = *impl_;
+    if (B != M.batch) const_cast<SparseOnnxModel *>(this)->resize_buffers(B);
+    if (!dInput || !dOutput) throw std::runtime_error("run_device: null device pointer");
+    std::lock_guard<std::mutex> lock(context_mutex());
+    if (M.layers.empty()) {
+        check(so_d2d(context(), dOutput, dInput, M.in_features * B * sizeof(float)), "so_d2d");
+        return;
+    }
+    M.enqueue_layers(dInput, dOutput);
+}
