@@ -1,0 +1,250 @@
+"""ctypes binding of the C ABI of libsparseops_hip.so (include/sparseops_hip.h).
+
+This is the stub a maintainer of a Python caller would write; the tests and the
+benchmark drive the HIP kernels through it with device-resident operands.
+"""
+import ctypes as ct
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "libsparseops_hip.so")
+
+SO_OK, SO_ERR_NO_DEVICE, SO_ERR_INVALID, SO_ERR_OOM, SO_ERR_HIP, SO_ERR_BOUNDS = range(6)
+ACT = {"none": 0, "relu": 1, "sigmoid": 2, "tanh": 3}
+LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS = 1, 2, 4
+
+# Every symbol include/sparseops_hip.h declares.
+SYMBOLS = (
+    "so_device_count so_init so_destroy so_last_error so_device_info so_malloc so_free so_h2d so_d2h "
+    "so_d2d so_fill_zero so_sync so_timer_begin so_timer_end so_ellpack_upload so_ellpack_free "
+    "so_ellpack_dims so_ellpack_download so_matmul so_matvec so_conv_plan_create so_conv_plan_free "
+    "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_graph_begin so_graph_end "
+    "so_graph_launch so_graph_free").split()
+
+_vp = ct.c_void_p
+_u32 = ct.c_uint32
+
+
+class ConvGeom(ct.Structure):
+    _fields_ = [(k, _u32) for k in (
+        "Cin", "Cout", "kH", "kW", "stride_h", "stride_w", "pad_h", "pad_w",
+        "dil_h", "dil_w", "H_in", "W_in", "H_out", "W_out")]
+
+
+class PoolGeom(ct.Structure):
+    _fields_ = [(k, _u32) for k in ("C", "H", "W", "H_out", "W_out")] + \
+               [(k, ct.c_int32) for k in ("kH", "kW", "sH", "sW", "padH0", "padW0")]
+
+
+def conv_geom(Cin, Cout, kH, kW, H, W, stride=(1, 1), pad=(0, 0), dil=(1, 1)):
+    Ho = (H + 2 * pad[0] - (dil[0] * (kH - 1) + 1)) // stride[0] + 1
+    Wo = (W + 2 * pad[1] - (dil[1] * (kW - 1) + 1)) // stride[1] + 1
+    return ConvGeom(Cin, Cout, kH, kW, stride[0], stride[1], pad[0], pad[1], dil[0], dil[1], H, W, Ho, Wo)
+
+
+class SoError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("so_status %d: %s" % (status, message))
+        self.status = status
+
+
+def load_library(path=None):
+    path = path or LIB_PATH
+    if not os.path.exists(path):
+        raise FileNotFoundError("libsparseops_hip.so is not built: %s (run __graft_entry__.build())" % path)
+    lib = ct.CDLL(path)
+    lib.so_last_error.restype = ct.c_char_p
+    sig = {
+        "so_device_count": [ct.POINTER(ct.c_int)],
+        "so_init": [ct.c_int, ct.POINTER(_vp)],
+        "so_destroy": [_vp],
+        "so_device_info": [_vp, ct.c_char_p, ct.c_size_t, ct.POINTER(ct.c_int)],
+        "so_malloc": [_vp, ct.c_size_t, ct.POINTER(_vp)],
+        "so_free": [_vp, _vp],
+        "so_h2d": [_vp, _vp, _vp, ct.c_size_t],
+        "so_d2h": [_vp, _vp, _vp, ct.c_size_t],
+        "so_d2d": [_vp, _vp, _vp, ct.c_size_t],
+        "so_fill_zero": [_vp, _vp, ct.c_size_t],
+        "so_sync": [_vp],
+        "so_timer_begin": [_vp],
+        "so_timer_end": [_vp, ct.POINTER(ct.c_float)],
+        "so_ellpack_upload": [_vp, _vp, _vp, _vp, _u32, _u32, _u32, ct.c_int, ct.POINTER(_vp)],
+        "so_ellpack_free": [_vp, _vp],
+        "so_ellpack_dims": [_vp, ct.POINTER(_u32), ct.POINTER(_u32), ct.POINTER(_u32),
+                            ct.POINTER(ct.c_uint64), ct.POINTER(ct.c_int)],
+        "so_ellpack_download": [_vp, _vp, ct.c_int, _vp, _vp, _vp],
+        "so_matmul": [_vp, _vp, _vp, _u32, _vp, _vp, ct.c_int],
+        "so_matvec": [_vp, _vp, _vp, _vp, _vp, ct.c_int],
+        "so_conv_plan_create": [_vp, _vp, ct.POINTER(ConvGeom), ct.POINTER(_vp)],
+        "so_conv_plan_free": [_vp, _vp],
+        "so_conv2d": [_vp, _vp, _vp, _u32, _vp, _vp, ct.c_int],
+        "so_maxpool": [_vp, ct.POINTER(PoolGeom), _vp, _u32, _vp],
+        "so_gap": [_vp, _u32, _u32, _u32, _vp, _u32, _vp],
+        "so_add": [_vp, _vp, _vp, ct.c_size_t, _vp],
+        "so_act": [_vp, ct.c_int, _vp, ct.c_size_t, _vp],
+        "so_transpose": [_vp, _vp, _u32, _u32, _vp],
+        "so_graph_begin": [_vp],
+        "so_graph_end": [_vp, ct.POINTER(_vp)],
+        "so_graph_launch": [_vp, _vp],
+        "so_graph_free": [_vp, _vp],
+    }
+    for name, argtypes in sig.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = ct.c_int
+    return lib
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(_vp)
+
+
+class DeviceArray:
+    """A float32/uint32 array in HBM, owned by a Context."""
+
+    def __init__(self, ctx, shape, dtype=np.float32):
+        self.ctx, self.shape, self.dtype = ctx, tuple(shape), np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+        p = _vp()
+        ctx._ck(ctx.lib.so_malloc(ctx.h, self.nbytes, ct.byref(p)))
+        self.ptr = p.value
+
+    def upload(self, host):
+        host = np.ascontiguousarray(host, dtype=self.dtype)
+        assert host.nbytes == self.nbytes, (host.shape, self.shape)
+        self.ctx._ck(self.ctx.lib.so_h2d(self.ctx.h, self.ptr, _ptr(host), self.nbytes))
+        return self
+
+    def download(self):
+        out = np.empty(self.shape, dtype=self.dtype)
+        self.ctx._ck(self.ctx.lib.so_d2h(self.ctx.h, _ptr(out), self.ptr, self.nbytes))
+        return out
+
+    def free(self):
+        if self.ptr:
+            self.ctx.lib.so_free(self.ctx.h, self.ptr)
+            self.ptr = None
+
+
+class DeviceEllpack:
+    def __init__(self, ctx, handle, m, n, r):
+        self.ctx, self.h, self.m, self.n, self.r = ctx, handle, m, n, r
+
+    def download(self, layout=LAYOUT_ROW):
+        shape = (self.m, self.r) if layout == LAYOUT_ROW else (self.r, self.m)
+        Wd = np.empty(shape, dtype=np.float32)
+        idx = np.empty(shape, dtype=np.uint32)
+        nnz = np.empty(self.m, dtype=np.uint32)
+        self.ctx._ck(self.ctx.lib.so_ellpack_download(self.ctx.h, self.h, layout, _ptr(Wd), _ptr(idx), _ptr(nnz)))
+        return Wd, idx, nnz
+
+    def free(self):
+        if self.h:
+            self.ctx.lib.so_ellpack_free(self.ctx.h, self.h)
+            self.h = None
+
+
+class Context:
+    """One so_ctx.  Raises SoError(SO_ERR_NO_DEVICE) when no GPU is usable."""
+
+    def __init__(self, device=0, lib=None):
+        self.lib = lib or load_library()
+        h = _vp()
+        self.h = None
+        self._ck(self.lib.so_init(device, ct.byref(h)))
+        self.h = h.value
+
+    def _ck(self, status):
+        if status != SO_OK:
+            raise SoError(status, self.lib.so_last_error().decode())
+
+    def close(self):
+        if self.h:
+            self.lib.so_destroy(self.h)
+            self.h = None
+
+    def info(self):
+        name = ct.create_string_buffer(64)
+        cus = ct.c_int()
+        self._ck(self.lib.so_device_info(self.h, name, 64, ct.byref(cus)))
+        return name.value.decode(), cus.value
+
+    def array(self, host, dtype=np.float32):
+        host = np.ascontiguousarray(host, dtype=dtype)
+        return DeviceArray(self, host.shape, dtype).upload(host)
+
+    def empty(self, shape, dtype=np.float32):
+        return DeviceArray(self, shape, dtype)
+
+    def sync(self):
+        self._ck(self.lib.so_sync(self.h))
+
+    def timer_begin(self):
+        self._ck(self.lib.so_timer_begin(self.h))
+
+    def timer_end(self):
+        ms = ct.c_float()
+        self._ck(self.lib.so_timer_end(self.h, ct.byref(ms)))
+        return ms.value
+
+    def upload_ellpack(self, Wd, idx, nnz, m, n, r, layouts=LAYOUT_ROW):
+        Wd = np.ascontiguousarray(Wd, dtype=np.float32)
+        idx = np.ascontiguousarray(idx, dtype=np.uint32)
+        nnz = np.ascontiguousarray(nnz, dtype=np.uint32)
+        h = _vp()
+        self._ck(self.lib.so_ellpack_upload(self.h, _ptr(Wd), _ptr(idx), _ptr(nnz), m, n, r, layouts, ct.byref(h)))
+        return DeviceEllpack(self, h.value, m, n, r)
+
+    def matmul(self, E, dX, C, dBias, dY, act="none"):
+        self._ck(self.lib.so_matmul(self.h, E.h, dX.ptr, C, dBias.ptr if dBias else None, dY.ptr, ACT[act]))
+
+    def matvec(self, E, dx, dBias, dy, layout=0):
+        self._ck(self.lib.so_matvec(self.h, E.h, dx.ptr, dBias.ptr if dBias else None, dy.ptr, layout))
+
+    def conv_plan(self, E, geom):
+        h = _vp()
+        self._ck(self.lib.so_conv_plan_create(self.h, E.h, ct.byref(geom), ct.byref(h)))
+        return h.value
+
+    def conv_plan_free(self, plan):
+        self.lib.so_conv_plan_free(self.h, plan)
+
+    def conv2d(self, plan, dX, B, dBias, dY, act="none"):
+        self._ck(self.lib.so_conv2d(self.h, plan, dX.ptr, B, dBias.ptr if dBias else None, dY.ptr, ACT[act]))
+
+    def maxpool(self, C, H, W, k, s, pad, dX, B, dY):
+        Ho = (H + 2 * pad[0] - k[0]) // s[0] + 1
+        Wo = (W + 2 * pad[1] - k[1]) // s[1] + 1
+        g = PoolGeom(C, H, W, Ho, Wo, k[0], k[1], s[0], s[1], pad[0], pad[1])
+        self._ck(self.lib.so_maxpool(self.h, ct.byref(g), dX.ptr, B, dY.ptr))
+
+    def gap(self, C, H, W, dX, B, dY):
+        self._ck(self.lib.so_gap(self.h, C, H, W, dX.ptr, B, dY.ptr))
+
+    def add(self, dA, dB, n, dD):
+        self._ck(self.lib.so_add(self.h, dA.ptr, dB.ptr, n, dD.ptr))
+
+    def act(self, act, dX, n, dY):
+        self._ck(self.lib.so_act(self.h, ACT[act], dX.ptr, n, dY.ptr))
+
+    def transpose(self, dSrc, rows, cols, dDst):
+        self._ck(self.lib.so_transpose(self.h, dSrc.ptr, rows, cols, dDst.ptr))
+
+    def fill_zero(self, dA):
+        self._ck(self.lib.so_fill_zero(self.h, dA.ptr, dA.nbytes))
+
+    def graph_begin(self):
+        self._ck(self.lib.so_graph_begin(self.h))
+
+    def graph_end(self):
+        g = _vp()
+        self._ck(self.lib.so_graph_end(self.h, ct.byref(g)))
+        return g.value
+
+    def graph_launch(self, g):
+        self._ck(self.lib.so_graph_launch(self.h, g))
+
+    def graph_free(self, g):
+        self.lib.so_graph_free(self.h, g)

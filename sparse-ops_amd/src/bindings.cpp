@@ -12,6 +12,7 @@
 #include "ellpack_encoder.hpp"
 #include "ellpack_matmul.hpp"
 #include "ellpack_matvec.hpp"
+#include "onnx_wire.hpp"
 #include "sparse_onnx.hpp"
 
 namespace py = pybind11;
@@ -103,6 +104,59 @@ PYBIND11_MODULE(sparseops_backend, mod)
     mod.def("device_available", []() {
         int n = 0;
         return so_device_count(&n) == SO_OK && n > 0;
+    });
+
+    // extension: what the built-in protobuf reader sees in an .onnx file (no device needed)
+    mod.def("parse_onnx", [](const std::string &path) {
+        const onnxwire::Model m = onnxwire::load_model(path);
+        py::dict out;
+        out["ir_version"] = m.ir_version;
+        out["producer_name"] = m.producer_name;
+        py::list opsets;
+        for (const auto &o : m.opset_import) opsets.append(py::make_tuple(o.first, o.second));
+        out["opset_import"] = opsets;
+        py::list nodes;
+        for (const auto &n : m.graph.node) {
+            py::dict d, attrs;
+            d["op_type"] = n.op_type;
+            d["name"] = n.name;
+            d["input"] = n.input;
+            d["output"] = n.output;
+            for (const auto &a : n.attribute) {
+                if (!a.ints.empty()) attrs[py::str(a.name)] = a.ints;
+                else if (!a.floats.empty()) attrs[py::str(a.name)] = a.floats;
+                else if (a.type == 1) attrs[py::str(a.name)] = a.f;
+                else if (a.type == 3) attrs[py::str(a.name)] = py::bytes(a.s);
+                else attrs[py::str(a.name)] = a.i;
+            }
+            d["attrs"] = attrs;
+            nodes.append(d);
+        }
+        out["nodes"] = nodes;
+        py::dict inits;
+        for (const auto &t : m.graph.initializer) {
+            std::vector<py::ssize_t> shape(t.dims.begin(), t.dims.end());
+            py::array_t<float> a(shape);
+            const std::vector<float> v = t.floats();
+            if (!v.empty()) std::memcpy(a.mutable_data(), v.data(), v.size() * sizeof(float));
+            inits[py::str(t.name)] = a;
+        }
+        out["initializers"] = inits;
+        auto vis = [](const std::vector<onnxwire::ValueInfo> &v) {
+            py::list l;
+            for (const auto &vi : v) {
+                py::list dims;
+                for (const auto &d : vi.dims) {
+                    if (d.has_value) dims.append(d.value);
+                    else dims.append(d.param);
+                }
+                l.append(py::make_tuple(vi.name, py::tuple(dims)));
+            }
+            return l;
+        };
+        out["inputs"] = vis(m.graph.input);
+        out["outputs"] = vis(m.graph.output);
+        return out;
     });
 
     py::class_<SparseOnnxModel>(mod, "SparseOnnxModel")

@@ -1,0 +1,163 @@
+"""so_conv2d (implicit im2col), so_maxpool, so_gap, so_add, so_act, so_transpose on
+the GPU against the oracle: bit-exact for everything whose arithmetic is fixed
+(conv with NONE/RELU, max, the ordered GAP sum, add, relu, transpose), 1e-6
+relative for the sigmoid/tanh library calls."""
+import numpy as np
+import pytest
+
+from conftest import as_oracle, rel_err, sparse_matrix
+
+import datagen
+import hipabi
+
+pytestmark = pytest.mark.gpu
+
+
+def gpu_conv(ctx, E, g, X, B, bias, act="none"):
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+    plan = ctx.conv_plan(dE, g)
+    dX, dY = ctx.array(X), ctx.empty((g.Cout, g.H_out, g.W_out, B))
+    dB = ctx.array(bias) if bias is not None else None
+    ctx.conv2d(plan, dX, B, dB, dY, act)
+    Y = dY.download()
+    ctx.conv_plan_free(plan)
+    dE.free()
+    return Y
+
+
+CASES = [(5, 7, 9, 11, 3, (3, 3), (1, 1), (1, 1), (1, 1)), (5, 7, 9, 11, 3, (3, 3), (2, 2), (1, 1), (1, 1)),
+         (8, 16, 14, 14, 32, (1, 1), (2, 2), (0, 0), (1, 1)), (3, 4, 10, 10, 5, (3, 2), (1, 2), (2, 0), (2, 1)),
+         (16, 32, 28, 28, 32, (3, 3), (1, 1), (1, 1), (1, 1)), (3, 64, 32, 32, 8, (7, 7), (2, 2), (3, 3), (1, 1)),
+         (4, 3, 6, 6, 1, (3, 3), (1, 1), (0, 0), (1, 1)), (2, 9, 5, 5, 64, (5, 5), (1, 1), (2, 2), (1, 1)),
+         (64, 64, 8, 8, 16, (3, 3), (1, 1), (1, 1), (1, 1))]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,Wi,B,k,s,p,d", CASES)
+def test_conv_bit_exact(ctx, oracle, Cin, Cout, H, Wi, B, k, s, p, d):
+    from oracle import conv_geom as ocg
+    rng = np.random.default_rng(Cin * 100 + H + B)
+    Wc = sparse_matrix(rng, Cout, Cin * k[0] * k[1], .7)
+    X = rng.standard_normal((Cin, H, Wi, B)).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    E = datagen.encode_dense(Wc)
+    g, og = hipabi.conv_geom(Cin, Cout, k[0], k[1], H, Wi, s, p, d), ocg(Cin, Cout, k[0], k[1], H, Wi, s, p, d)
+    for act in ("none", "relu"):
+        for bias in (b, None):
+            assert np.array_equal(gpu_conv(ctx, E, g, X, B, bias, act), oracle.conv2d_pf(as_oracle(E), og, X, B, bias, act))
+    for act in ("sigmoid", "tanh"):
+        assert rel_err(gpu_conv(ctx, E, g, X, B, b, act), oracle.conv2d_pf(as_oracle(E), og, X, B, b, act)) <= 1e-6
+
+
+def test_conv_reference_vectors(ctx, golden):
+    for i, c in enumerate(golden["conv_cases"]):
+        Cin, Cout, H, Wi, B = (int(v) for v in c[:5])
+        k, s, p, d = [tuple(int(v) for v in c[j:j + 2]) for j in (5, 7, 9, 11)]
+        g = hipabi.conv_geom(Cin, Cout, k[0], k[1], H, Wi, s, p, d)
+        E = datagen.encode_dense(golden["conv%d_W" % i])
+        X, b = golden["conv%d_X" % i], golden["conv%d_b" % i]
+        assert np.array_equal(gpu_conv(ctx, E, g, X, B, b), golden["conv%d_Y" % i])
+        assert np.array_equal(gpu_conv(ctx, E, g, X, B, b, "relu"), golden["conv%d_Yrelu" % i])
+
+
+def test_conv_special_cases(ctx, oracle):
+    rng = np.random.default_rng(12)
+    Cin, Cout, H, Wi, B = 6, 5, 7, 9, 4
+    X = rng.standard_normal((Cin, H, Wi, B)).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    W = sparse_matrix(rng, Cout, Cin, .4)
+    E = datagen.encode_dense(W)
+    # 1x1 conv == so_matmul on [Cin x H*W*B], bit for bit
+    Y = gpu_conv(ctx, E, hipabi.conv_geom(Cin, Cout, 1, 1, H, Wi), X, B, b)
+    assert np.array_equal(Y.reshape(Cout, -1), oracle.matmul(as_oracle(E), X.reshape(Cin, -1), b))
+    # delta kernel at the centre of a padded 3x3 is the identity
+    W4 = np.zeros((Cin, Cin, 3, 3), np.float32)
+    W4[np.arange(Cin), np.arange(Cin), 1, 1] = 1
+    Y = gpu_conv(ctx, datagen.encode_dense(W4.reshape(Cin, -1)), hipabi.conv_geom(Cin, Cin, 3, 3, H, Wi, pad=(1, 1)), X, B, None)
+    assert np.array_equal(Y, X)
+    # padding taps are skipped, not multiplied: inf at the border must not leak NaN through zero weights
+    Xi = X.copy()
+    Xi[:, 0, 0, :] = np.inf
+    Y = gpu_conv(ctx, datagen.encode_dense(W4.reshape(Cin, -1)), hipabi.conv_geom(Cin, Cin, 3, 3, H, Wi, pad=(1, 1)), Xi, B, None)
+    assert np.array_equal(Y, Xi)
+
+
+def test_conv_plan_validation(ctx):
+    E = datagen.encode_dense(np.ones((4, 18), np.float32))
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+    g = hipabi.conv_geom(2, 4, 3, 3, 8, 8)
+    bad = hipabi.conv_geom(3, 4, 3, 3, 8, 8)             # K mismatch
+    with pytest.raises(hipabi.SoError):
+        ctx.conv_plan(dE, bad)
+    wrong = hipabi.conv_geom(2, 4, 3, 3, 8, 8)
+    wrong.H_out = 7                                       # not the loader's formula
+    with pytest.raises(hipabi.SoError):
+        ctx.conv_plan(dE, wrong)
+    ctx.conv_plan_free(ctx.conv_plan(dE, g))
+    dE.free()
+
+
+@pytest.mark.parametrize("C,H,Wi,B,k,s,p", [(3, 8, 8, 2, (2, 2), (2, 2), (0, 0)), (4, 9, 7, 3, (3, 3), (2, 2), (1, 1)),
+                                           (2, 5, 6, 1, (3, 2), (1, 1), (1, 0)), (64, 56, 56, 8, (3, 3), (2, 2), (1, 1))])
+def test_maxpool(ctx, oracle, C, H, Wi, B, k, s, p):
+    rng = np.random.default_rng(C + H)
+    X = rng.standard_normal((C, H, Wi, B)).astype(np.float32)
+    Yo = oracle.maxpool_pf(X, C, H, Wi, B, k, s, p)
+    dY = ctx.empty(Yo.shape)
+    ctx.maxpool(C, H, Wi, k, s, p, ctx.array(X), B, dY)
+    assert np.array_equal(dY.download(), Yo)
+
+
+def test_gap_add_act_transpose(ctx, oracle):
+    rng = np.random.default_rng(3)
+    C, H, Wi, B = 37, 7, 6, 33
+    X = rng.standard_normal((C, H, Wi, B)).astype(np.float32)
+    dX = ctx.array(X)
+    Yo = oracle.gap_pf(X, C, H, Wi, B)
+    dY = ctx.empty(Yo.shape)
+    ctx.gap(C, H, Wi, dX, B, dY)
+    assert np.array_equal(dY.download(), Yo)
+    A = rng.standard_normal(X.shape).astype(np.float32)
+    dA, dD = ctx.array(A), ctx.empty(X.shape)
+    ctx.add(dX, dA, X.size, dD)
+    assert np.array_equal(dD.download(), oracle.add(X, A))
+    ctx.add(dX, dA, X.size, dA)                          # in place on an operand
+    assert np.array_equal(dA.download(), X + A)
+    V = (rng.standard_normal(100003) * 4).astype(np.float32)
+    dV, dO = ctx.array(V), ctx.empty(V.shape)
+    for act in ("none", "relu", "sigmoid", "tanh"):
+        ctx.act(act, dV, V.size, dO)
+        if act in ("none", "relu"):
+            assert np.array_equal(dO.download(), oracle.act(V, act))
+        else:
+            assert rel_err(dO.download(), oracle.act(V, act)) <= 1e-6
+    for (r, c) in [(70, 130), (1, 1), (64, 64), (32, 150528 // 64), (1000, 3)]:
+        S = rng.standard_normal((r, c)).astype(np.float32)
+        dT = ctx.empty((c, r))
+        ctx.transpose(ctx.array(S), r, c, dT)
+        assert np.array_equal(dT.download(), S.T)
+
+
+def test_launch_graph_replays(ctx, oracle):
+    """A recorded chain replays with the same bits as eager execution, several
+    times, with eager work and synchronisation in between."""
+    rng = np.random.default_rng(21)
+    W1, W2 = sparse_matrix(rng, 96, 64, .8), sparse_matrix(rng, 40, 96, .8)
+    E1, E2 = datagen.encode_dense(W1), datagen.encode_dense(W2)
+    d1 = ctx.upload_ellpack(E1.Wd, E1.idx, E1.nnz, E1.m, E1.n, E1.r)
+    d2 = ctx.upload_ellpack(E2.Wd, E2.idx, E2.nnz, E2.m, E2.n, E2.r)
+    C = 48
+    dX, dH, dY = ctx.empty((64, C)), ctx.empty((96, C)), ctx.empty((40, C))
+    ctx.graph_begin()
+    ctx.matmul(d1, dX, C, None, dH, "relu")
+    ctx.matmul(d2, dH, C, None, dY, "none")
+    g = ctx.graph_end()
+    for it in range(4):
+        X = rng.standard_normal((64, C)).astype(np.float32)
+        dX.upload(X)
+        ctx.fill_zero(dY)
+        ctx.sync()
+        ctx.graph_launch(g)
+        Y = dY.download()
+        Yo = oracle.matmul(as_oracle(E2), oracle.matmul(as_oracle(E1), X, None, "relu"), None)
+        assert np.array_equal(Y, Yo), it
+    ctx.graph_free(g)

@@ -1,0 +1,163 @@
+"""so_matmul (C ABI) and sparseops_backend.ellpack_matmul on the GPU against the
+oracle.  NONE/RELU epilogues must be bit-identical to the oracle (same rounding
+sequence: bias, then one FMA per stored nonzero in ascending slot order);
+SIGMOID/TANH use the device's expf/tanhf and must agree to 1e-6 relative."""
+import numpy as np
+import pytest
+
+from conftest import as_oracle, rel_err, sparse_matrix
+from test_oracle_kernels import MATMUL_CASES
+
+import datagen
+import hipabi
+
+pytestmark = pytest.mark.gpu
+ACT_TOL = 1e-6
+
+
+def gpu_matmul(ctx, E, X, bias, act="none"):
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+    dX, dY = ctx.array(X), ctx.empty((E.m, X.shape[1]))
+    dB = ctx.array(bias) if bias is not None else None
+    ctx.matmul(dE, dX, X.shape[1], dB, dY, act)
+    Y = dY.download()
+    for a in (dX, dY, dB):
+        if a is not None:
+            a.free()
+    dE.free()
+    return Y
+
+
+@pytest.mark.parametrize("m,n,C,sp", MATMUL_CASES + [(64, 96, 16, .5), (64, 96, 64, .5), (64, 96, 128, .5),
+                                                     (64, 96, 192, .5), (64, 96, 256, .5), (64, 96, 320, .5),
+                                                     (64, 96, 512, .8), (64, 96, 1024, .8), (7, 9, 65, .3),
+                                                     (130, 70, 129, .6), (2000, 2000, 10, .3), (3000, 3000, 10, .4)])
+def test_matmul_bit_exact(ctx, oracle, m, n, C, sp):
+    rng = np.random.default_rng(m * 31 + n * 7 + C)
+    W = sparse_matrix(rng, m, n, sp)
+    X = rng.standard_normal((n, C)).astype(np.float32)
+    b = rng.standard_normal(m).astype(np.float32)
+    E = datagen.encode_dense(W)
+    Y = gpu_matmul(ctx, E, X, b)
+    assert Y.shape == (m, C)
+    assert np.array_equal(Y, oracle.matmul(as_oracle(E), X, b))
+    if m and C:
+        assert rel_err(Y, W.astype(np.float64) @ X + b[:, None].astype(np.float64)) <= 1e-5
+        # the reference's own assertion (tests/unit/test_matmul.py:48)
+        assert np.allclose(Y, W @ X + b[:, None], atol=1e-5 * max(1.0, np.abs(Y).max()))
+
+
+@pytest.mark.parametrize("C", [1, 10, 64, 100, 128, 256, 300])
+@pytest.mark.parametrize("act", ["none", "relu", "sigmoid", "tanh"])
+def test_matmul_epilogues(ctx, oracle, C, act):
+    rng = np.random.default_rng(C)
+    W = sparse_matrix(rng, 150, 200, .85)
+    X = rng.standard_normal((200, C)).astype(np.float32)
+    b = rng.standard_normal(150).astype(np.float32)
+    E = datagen.encode_dense(W)
+    for bias in (b, None):
+        Y, Yo = gpu_matmul(ctx, E, X, bias, act), oracle.matmul(as_oracle(E), X, bias, act)
+        if act in ("none", "relu"):
+            assert np.array_equal(Y, Yo)
+        else:
+            assert rel_err(Y, Yo) <= ACT_TOL
+
+
+def test_matmul_reference_vectors(ctx, golden):
+    E = datagen.encode_dense(golden["enc_W"])
+    b = golden["mm_bias"]
+    for C in (1, 10, 16, 64, 100, 128, 256):
+        X = golden["mm_X_%d" % C]
+        assert np.array_equal(gpu_matmul(ctx, E, X, b), golden["mm_Y_%d" % C])
+        assert np.array_equal(gpu_matmul(ctx, E, X, b, "relu"), golden["mm_Yrelu_%d" % C])
+    assert np.array_equal(gpu_matmul(ctx, E, golden["mm_X_64"], None), golden["mm_Ynobias_64"])
+
+
+def test_matmul_config1_and_config3(ctx, oracle):
+    E, X, b, W = datagen.config1()
+    assert abs(E.r - 133) < 20 and abs(E.total_nnz - 104858) < 2000
+    Y = gpu_matmul(ctx, E, X, b)
+    assert np.array_equal(Y, oracle.matmul(as_oracle(E), X, b))
+    assert rel_err(Y, W.astype(np.float64) @ X + b[:, None]) <= 1e-5
+    E, X, b = datagen.config3()
+    assert E.r == 410 and E.total_nnz == 4096 * 410 and (E.nnz == 410).all()
+    Y = gpu_matmul(ctx, E, X, b)
+    assert np.array_equal(Y, oracle.matmul(as_oracle(E), X, b))
+    # size-independent properties at full size: every column is computed
+    # independently of the tiling, so one column alone gives the same bits ...
+    for c in (0, 77, 255):
+        assert np.array_equal(gpu_matmul(ctx, E, np.ascontiguousarray(X[:, c:c + 1]), b)[:, 0], Y[:, c])
+    # ... and a permutation of X's columns permutes Y's columns
+    perm = np.random.default_rng(0).permutation(256)
+    assert np.array_equal(gpu_matmul(ctx, E, np.ascontiguousarray(X[:, perm]), b), Y[:, perm])
+
+
+def test_matmul_degenerate_shapes(ctx, oracle):
+    # zero-sized launches are early-outs, not HIP errors
+    for (m, n, C) in [(0, 0, 0), (0, 5, 3), (5, 0, 3), (5, 4, 0)]:
+        W = np.ones((m, n), np.float32)
+        E = datagen.encode_dense(W)
+        b = np.arange(m, dtype=np.float32)
+        Y = gpu_matmul(ctx, E, np.ones((n, C), np.float32), b)
+        assert Y.shape == (m, C)
+        if Y.size:
+            assert np.array_equal(Y, np.repeat(b[:, None], C, axis=1))     # r = 0: bias only
+    E = datagen.encode_dense(np.zeros((32, 32), np.float32))              # all-zero matrix, r = 0
+    assert E.r == 0
+    assert np.array_equal(gpu_matmul(ctx, E, np.ones((32, 7), np.float32), None), np.zeros((32, 7), np.float32))
+
+
+def test_matmul_padding_is_not_read(ctx):
+    """0 * inf = NaN: a kernel that streamed padded slots (Wd = 0, idx = 0) would
+    poison rows shorter than r when X[0, :] is infinite."""
+    W = np.zeros((4, 6), np.float32)
+    W[0, 1:5] = 1
+    W[1, 2] = 2
+    X = np.ones((6, 70), np.float32)
+    X[0, :] = np.inf
+    Y = gpu_matmul(ctx, datagen.encode_dense(W), X, None)
+    assert np.isfinite(Y).all() and np.array_equal(Y[:, 0], [4, 2, 0, 0])
+
+
+def test_upload_validation_and_layout_round_trip(ctx):
+    rng = np.random.default_rng(4)
+    E = datagen.encode_dense(sparse_matrix(rng, 50, 70, .8))
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, hipabi.LAYOUT_ROW | hipabi.LAYOUT_SLOT | hipabi.LAYOUT_BINS)
+    Wd, idx, nnz = dE.download(hipabi.LAYOUT_ROW)
+    assert np.array_equal(Wd, E.Wd) and np.array_equal(idx, E.idx) and np.array_equal(nnz, E.nnz)
+    WdT, idxT, _ = dE.download(hipabi.LAYOUT_SLOT)                       # slot-major: WdT[k*m+i] == Wd[i*r+k]
+    assert np.array_equal(WdT, E.Wd.T) and np.array_equal(idxT, E.idx.T)
+    dE.free()
+    bad = E.idx.copy()
+    bad[3, 0] = 70
+    with pytest.raises(hipabi.SoError) as e:
+        ctx.upload_ellpack(E.Wd, bad, E.nnz, E.m, E.n, E.r)
+    assert e.value.status == hipabi.SO_ERR_BOUNDS
+    badn = E.nnz.copy()
+    badn[0] = E.r + 1
+    with pytest.raises(hipabi.SoError) as e:
+        ctx.upload_ellpack(E.Wd, E.idx, badn, E.m, E.n, E.r)
+    assert e.value.status == hipabi.SO_ERR_BOUNDS
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+    with pytest.raises(hipabi.SoError):
+        dE.download(hipabi.LAYOUT_SLOT)                                   # not uploaded
+    dE.free()
+
+
+# ---- the drop-in module: the reference's own unit cases (tests/unit/test_matmul.py:12-48), seeded
+
+@pytest.mark.parametrize("m,n,C,sp", MATMUL_CASES)
+def test_backend_matmul(backend, oracle, m, n, C, sp):
+    rng = np.random.default_rng(m + n + C)
+    W = sparse_matrix(rng, m, n, sp, signed=False)
+    E = backend.convert_to_ellpack(W)
+    X = rng.random((n, C)).astype(np.float32)
+    b = rng.random(m).astype(np.float32)
+    y = backend.ellpack_matmul(E, X, b)
+    assert y.shape == (m, C)
+    assert np.allclose(y, W @ X + np.expand_dims(b, axis=1), atol=1e-5)
+    assert np.array_equal(y, oracle.matmul(oracle.encode(W), X, b))
+    if m and C:
+        assert np.array_equal(backend.ellpack_matmul(E, X, None), oracle.matmul(oracle.encode(W), X, None))
+        # non-contiguous / float64 inputs are force-cast like the reference does (src/bindings.cpp:112-113)
+        assert np.array_equal(backend.ellpack_matmul(E, np.asfortranarray(X).astype(np.float64), b), y)

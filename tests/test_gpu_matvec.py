@@ -1,0 +1,145 @@
+"""so_matvec (all three device layouts) and sparseops_backend.ellpack_matvec on the
+GPU.  The in-row summation order differs from the reference's (wave reduction vs.
+16 interleaved partials), so the bar is the fp32 tolerance: max|y - ref| / max|ref|
+<= 1e-5 against both the fp64 product and the oracle."""
+import numpy as np
+import pytest
+
+from conftest import as_oracle, rel_err, sparse_matrix
+from test_oracle_kernels import MATVEC_CASES
+
+import datagen
+import hipabi
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+ALL = hipabi.LAYOUT_ROW | hipabi.LAYOUT_SLOT | hipabi.LAYOUT_BINS
+
+
+def gpu_matvec(ctx, E, x, bias, layouts=ALL, which=(hipabi.LAYOUT_ROW, hipabi.LAYOUT_SLOT, hipabi.LAYOUT_BINS, 0)):
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, layouts)
+    dx, dy = ctx.array(x), ctx.empty((E.m,))
+    dB = ctx.array(bias) if bias is not None else None
+    out = {}
+    for lay in which:
+        dy.upload(np.full(E.m, np.nan, np.float32))      # every row must be written
+        ctx.matvec(dE, dx, dB, dy, lay)
+        out[lay] = dy.download()
+    dE.free()
+    return out
+
+
+@pytest.mark.parametrize("m,n,sp", MATVEC_CASES + [(257, 4097, .5), (5000, 64, .2), (100, 50000, .99)])
+def test_matvec_all_layouts(ctx, oracle, m, n, sp):
+    rng = np.random.default_rng(m * 13 + n)
+    W = sparse_matrix(rng, m, n, sp)
+    x = rng.standard_normal(n).astype(np.float32)
+    b = rng.standard_normal(m).astype(np.float32)
+    E = datagen.encode_dense(W)
+    y64 = W.astype(np.float64) @ x + b
+    yo = oracle.matvec(as_oracle(E), x, b)
+    for lay, y in gpu_matvec(ctx, E, x, b).items():
+        assert y.shape == (m,)
+        assert rel_err(y, y64) <= TOL, lay
+        assert rel_err(y, yo) <= TOL, lay
+    for lay, y in gpu_matvec(ctx, E, x, None, which=(hipabi.LAYOUT_ROW, hipabi.LAYOUT_BINS)).items():
+        assert rel_err(y, W.astype(np.float64) @ x) <= TOL, lay
+
+
+def test_matvec_every_row_written_once(ctx):
+    """Binned launches must cover every row exactly once: y starts as NaN."""
+    rng = np.random.default_rng(3)
+    counts = np.minimum(rng.zipf(1.3, size=3000), 400)
+    n = 1000
+    cols = [np.sort(rng.permutation(n)[:k]).astype(np.uint32) for k in counts]
+    vals = [rng.standard_normal(k).astype(np.float32) for k in counts]
+    E = datagen.rows_to_ellpack(3000, n, cols, vals)
+    x = rng.standard_normal(n).astype(np.float32)
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, ALL)
+    dx = ctx.array(x)
+    W = np.zeros((3000, n))
+    for i in range(3000):
+        W[i, cols[i]] = vals[i]
+    for lay in (hipabi.LAYOUT_ROW, hipabi.LAYOUT_SLOT, hipabi.LAYOUT_BINS):
+        dy = ctx.array(np.full(3000, np.nan, np.float32))
+        ctx.matvec(dE, dx, None, dy, lay)
+        y = dy.download()
+        assert np.isfinite(y).all(), lay
+        assert rel_err(y, W @ x) <= TOL, lay
+
+
+def test_matvec_reference_vectors(ctx, golden):
+    E = datagen.encode_dense(golden["enc_W"])
+    for lay, y in gpu_matvec(ctx, E, golden["mv_x"], golden["mm_bias"]).items():
+        assert rel_err(y, golden["mv_y"]) <= TOL, lay
+
+
+def test_matvec_padding_is_not_read(ctx):
+    W = np.zeros((5, 8), np.float32)
+    W[0, 1:7] = 1
+    W[2, 3] = 2
+    x = np.ones(8, np.float32)
+    x[0] = np.inf
+    for lay, y in gpu_matvec(ctx, datagen.encode_dense(W), x, None).items():
+        assert np.array_equal(y, [6, 0, 2, 0, 0]), lay
+
+
+def test_matvec_config2a_and_2b(ctx, oracle):
+    """Full-size configurations: 16384 x 16384 at 95 % uniform sparsity, and the
+    skewed variant with Zipf(1.2) row lengths clipped at 2048."""
+    E, x, b = datagen.config2a()
+    assert 880 < E.r < 1000 and abs(E.total_nnz - 0.05 * 16384 ** 2) < 5e4
+    yo = oracle.matvec(as_oracle(E), x, b)
+    for lay, y in gpu_matvec(ctx, E, x, b, layouts=hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS,
+                             which=(hipabi.LAYOUT_ROW, hipabi.LAYOUT_BINS)).items():
+        assert rel_err(y, yo) <= TOL, lay
+    E, x, b = datagen.config2b()
+    assert E.r == 2048 and E.total_nnz < E.m * E.r // 3
+    yo = oracle.matvec(as_oracle(E), x, b)
+    for lay, y in gpu_matvec(ctx, E, x, b, layouts=hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS,
+                             which=(hipabi.LAYOUT_ROW, hipabi.LAYOUT_BINS, 0)).items():
+        assert rel_err(y, yo) <= TOL, lay
+    # linearity in x is size-independent: E(2x) = 2 E(x) exactly (scaling by 2 is exact in fp32)
+    y1 = gpu_matvec(ctx, E, x, None, layouts=hipabi.LAYOUT_BINS, which=(hipabi.LAYOUT_BINS,))[hipabi.LAYOUT_BINS]
+    y2 = gpu_matvec(ctx, E, 2 * x, None, layouts=hipabi.LAYOUT_BINS, which=(hipabi.LAYOUT_BINS,))[hipabi.LAYOUT_BINS]
+    assert np.array_equal(y2, 2 * y1)
+
+
+def test_matvec_degenerate(ctx):
+    E = datagen.encode_dense(np.zeros((0, 0), np.float32))
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, 0, 0, 0, ALL)
+    ctx.matvec(dE, ctx.empty((0,)), None, ctx.empty((0,)), 0)          # no launch, no error
+    E = datagen.encode_dense(np.zeros((32, 32), np.float32))
+    b = np.arange(32, dtype=np.float32)
+    for lay, y in gpu_matvec(ctx, E, np.ones(32, np.float32), b).items():
+        assert np.array_equal(y, b), lay
+    with pytest.raises(hipabi.SoError):
+        dE2 = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, 32, 32, 0, hipabi.LAYOUT_ROW)
+        ctx.matvec(dE2, ctx.empty((32,)), None, ctx.empty((32,)), hipabi.LAYOUT_SLOT)   # layout not uploaded
+
+
+# ---- the drop-in module: the reference's unit cases (tests/unit/test_matvec.py:12-46), seeded
+
+@pytest.mark.parametrize("m,n,sp", MATVEC_CASES)
+def test_backend_matvec(backend, m, n, sp):
+    rng = np.random.default_rng(m + n)
+    W = sparse_matrix(rng, m, n, sp, signed=False)
+    E = backend.convert_to_ellpack(W)
+    x = rng.random(n).astype(np.float32)
+    b = rng.random(m).astype(np.float32)
+    y = backend.ellpack_matvec(E, x, b)
+    assert y.shape == (m,)
+    y64 = W.astype(np.float64) @ x + b
+    assert rel_err(y, y64) <= TOL
+    assert np.allclose(y, y64, rtol=1e-5, atol=1e-5 * max(1.0, np.abs(y64).max() if m else 1.0))
+    if m:
+        assert rel_err(backend.ellpack_matvec(E, x, None), W.astype(np.float64) @ x) <= TOL
+
+
+def test_backend_matvec_skewed(backend):
+    rng = np.random.default_rng(11)
+    W = sparse_matrix(rng, 800, 900, .995)
+    W[7] = rng.standard_normal(900)                 # one dense row: r = 900, mean nnz ~ 5
+    E = backend.convert_to_ellpack(W)
+    x = rng.standard_normal(900).astype(np.float32)
+    assert rel_err(backend.ellpack_matvec(E, x, None), W.astype(np.float64) @ x) <= TOL

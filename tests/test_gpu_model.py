@@ -1,0 +1,196 @@
+"""SparseOnnxModel on the GPU: ONNX graphs written by python/onnx_wire.py, executed
+by the device-resident layer chain, checked layer-composition-wise against the
+oracle (bit-exact where every layer is, 1e-5 relative otherwise) and against
+torch on the CPU (the reference's own comparisons use atol=1e-4,
+tests/test_onnx.py:135, tests/full_test.py:88)."""
+import os
+
+import numpy as np
+import pytest
+
+from conftest import rel_err
+
+import datagen
+import onnx_wire as ow
+
+pytestmark = pytest.mark.gpu
+ACTS = {"Relu": "relu", "Sigmoid": "sigmoid", "Tanh": "tanh", None: "none"}
+
+
+def oracle_mlp(oracle, Ws, acts, X_bm, biases=None):
+    """X_bm is (B, features); the chain runs on [features x B]."""
+    A = np.ascontiguousarray(X_bm.T)
+    for l, W in enumerate(Ws):
+        A = oracle.matmul(oracle.encode(W), A, None if biases is None else biases[l], ACTS[acts[l]])
+    return np.ascontiguousarray(A.T)
+
+
+@pytest.mark.parametrize("use_gemm", [False, True])
+def test_mlp_small(backend, oracle, tmp_path, use_gemm):
+    rng = np.random.default_rng(5)
+    dims, B = (37, 64, 50, 11), 24
+    Ws = [datagen.magnitude_prune(rng.standard_normal((o, i)).astype(np.float32), .8) for i, o in zip(dims[:-1], dims[1:])]
+    bs = [rng.standard_normal(o).astype(np.float32) for o in dims[1:]] if use_gemm else None
+    acts = ["Relu", "Sigmoid", None]
+    path = ow.save(str(tmp_path / "mlp.onnx"), ow.mlp_model(Ws, acts, B, bs, use_gemm))
+    model = backend.SparseOnnxModel(path)
+    assert model.output_shape() == [B, 11] and model.input_shape() == [B, 37]
+    desc = model.describe()
+    assert len(desc) == 3 and "act=relu" in desc[0] and "act=sigmoid" in desc[1] and "act=none" in desc[2]   # fused
+    X = rng.random((B, 37)).astype(np.float32)
+    Yo = oracle_mlp(oracle, Ws, acts, X, bs)
+    Y = model.run(X)                                      # C-order (B, F): transposed on the device
+    assert Y.shape == (B, 11) and rel_err(Y, Yo) <= 1e-6
+    Yf = model.run(np.asfortranarray(X))                  # Fortran order is already [F x B]
+    assert Yf.shape == (B, 11) and np.array_equal(Yf, Y)
+    assert np.array_equal(model.run(X.astype(np.float64)), Y)
+    # fp64 ground truth
+    A = X.astype(np.float64)
+    for l, W in enumerate(Ws):
+        A = A @ W.T.astype(np.float64) + (0 if bs is None else bs[l])
+        A = {"Relu": lambda v: np.maximum(v, 0), "Sigmoid": lambda v: 1 / (1 + np.exp(-v)), None: lambda v: v}[acts[l]](A)
+    assert rel_err(Y, A) <= 1e-5 and np.allclose(Y, A, atol=1e-4)
+
+
+def test_mlp_resize_and_repeat(backend, oracle, tmp_path):
+    rng = np.random.default_rng(6)
+    Ws = [datagen.magnitude_prune(rng.standard_normal((48, 30)).astype(np.float32), .7),
+          datagen.magnitude_prune(rng.standard_normal((9, 48)).astype(np.float32), .5)]
+    acts = ["Tanh", "Relu"]
+    model = backend.SparseOnnxModel(ow.save(str(tmp_path / "m.onnx"), ow.mlp_model(Ws, acts, 16)))
+    for B in (16, 16, 5, 64, 16, 1):
+        if B == 64:
+            model.resize_buffers(64)
+            assert model.batch() == 64
+        X = rng.standard_normal((B, 30)).astype(np.float32)
+        Y = model.run(X)
+        assert model.batch() == B and model.output_shape() == [B, 9]
+        assert rel_err(Y, oracle_mlp(oracle, Ws, acts, X)) <= 1e-6
+    with pytest.raises(RuntimeError, match="features per sample"):
+        model.run(np.zeros((4, 31), np.float32))
+
+
+def test_mlp_graph_and_eager_agree(backend, tmp_path):
+    rng = np.random.default_rng(7)
+    Ws = [datagen.magnitude_prune(rng.standard_normal((80, 60)).astype(np.float32), .8),
+          datagen.magnitude_prune(rng.standard_normal((20, 80)).astype(np.float32), .8)]
+    path = ow.save(str(tmp_path / "m.onnx"), ow.mlp_model(Ws, ["Relu", "Tanh"], 32))
+    X = rng.standard_normal((32, 60)).astype(np.float32)
+    Yg = backend.SparseOnnxModel(path).run(X)
+    os.environ["SPARSEOPS_NO_GRAPH"] = "1"
+    try:
+        Ye = backend.SparseOnnxModel(path).run(X)
+    finally:
+        del os.environ["SPARSEOPS_NO_GRAPH"]
+    assert np.array_equal(Yg, Ye)
+
+
+def test_mlp_config4(backend, oracle, tmp_path):
+    """784 -> 4096 -> 4096 -> 4096 -> 10, 90 % magnitude-pruned, ReLU/Sigmoid/Tanh, B = 256."""
+    Ws = datagen.config4_weights()
+    acts = ["Relu", "Sigmoid", "Tanh", None]
+    X = datagen.config4_input()
+    model = backend.SparseOnnxModel(ow.save(str(tmp_path / "c4.onnx"), ow.mlp_model(Ws, acts, 256)))
+    desc = model.describe()
+    assert len(desc) == 4 and all(d.startswith("MatMul") for d in desc)
+    Y = model.run(X)
+    Yo = oracle_mlp(oracle, Ws, acts, X)
+    assert Y.shape == (256, 10)
+    assert rel_err(Y, Yo) <= 1e-5 and np.allclose(Y, Yo, atol=1e-4)
+    assert np.array_equal(model.run(X), Y)               # deterministic across replays
+
+
+def cnn_model(rng, B, H=16):
+    """The reference's full_test.py topology (tests/full_test.py:21-41):
+    Conv3x3 -> ReLU -> MaxPool -> {Conv3x3 -> ReLU, Conv1x1} -> Add -> GAP -> Flatten -> FC -> ReLU,
+    plus a stride-2 conv and an Identity to exercise aliasing."""
+    t = {"W1": datagen.he_sparse_conv(rng, 8, 3, 3, .5), "b1": rng.standard_normal(8).astype(np.float32),
+         "W2": datagen.he_sparse_conv(rng, 16, 8, 3, .7), "b2": rng.standard_normal(16).astype(np.float32),
+         "W3": datagen.he_sparse_conv(rng, 16, 8, 1, .3),
+         "Wf": datagen.magnitude_prune(rng.standard_normal((10, 16)).astype(np.float32), .5),
+         "bf": rng.standard_normal(10).astype(np.float32)}
+    nodes = [ow.node("Conv", ["x", "W1", "b1"], ["c1"], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1]),
+             ow.node("Relu", ["c1"], ["r1"]),
+             ow.node("MaxPool", ["r1"], ["p1"], kernel_shape=[3, 3], strides=[2, 2], pads=[1, 1, 1, 1]),
+             ow.node("Identity", ["p1"], ["p1i"]),
+             ow.node("Conv", ["p1i", "W2", "b2"], ["c2"], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[2, 2]),
+             ow.node("Relu", ["c2"], ["r2"]),
+             ow.node("Conv", ["p1", "W3"], ["c3"], kernel_shape=[1, 1], strides=[2, 2]),
+             ow.node("Add", ["r2", "c3"], ["a1"]),
+             ow.node("GlobalAveragePool", ["a1"], ["g1"]),
+             ow.node("Flatten", ["g1"], ["f1"], axis=1),
+             ow.node("Gemm", ["f1", "Wf", "bf"], ["fc"], alpha=1.0, beta=1.0, transB=1),
+             ow.node("Relu", ["fc"], ["y"])]
+    return ow.model(nodes, [("x", (B, 3, H, H))], [("y", (B, 10))], list(t.items())), t
+
+
+def torch_cnn(t, X):
+    import torch
+    import torch.nn.functional as F
+    T = {k: torch.from_numpy(v).double() for k, v in t.items()}
+    x = torch.from_numpy(X).double()
+    p1 = F.max_pool2d(F.relu(F.conv2d(x, T["W1"], T["b1"], padding=1)), 3, 2, 1)
+    a1 = F.relu(F.conv2d(p1, T["W2"], T["b2"], stride=2, padding=1)) + F.conv2d(p1, T["W3"], None, stride=2)
+    return F.relu(a1.mean(dim=(2, 3)) @ T["Wf"].T + T["bf"]).numpy()
+
+
+def oracle_cnn(oracle, t, X):
+    from oracle import conv_geom
+    B, _, H, _ = X.shape
+    A = np.ascontiguousarray(X.transpose(1, 2, 3, 0))                        # [C][H][W][B]
+    E1, E2, E3 = (oracle.encode(t[k].reshape(t[k].shape[0], -1)) for k in ("W1", "W2", "W3"))
+    c1 = oracle.conv2d_pf(E1, conv_geom(3, 8, 3, 3, H, H, pad=(1, 1)), A, B, t["b1"], "relu")
+    p1 = oracle.maxpool_pf(c1, 8, H, H, B, (3, 3), (2, 2), (1, 1))
+    Hp = p1.shape[1]
+    r2 = oracle.conv2d_pf(E2, conv_geom(8, 16, 3, 3, Hp, Hp, (2, 2), (1, 1)), p1, B, t["b2"], "relu")
+    c3 = oracle.conv2d_pf(E3, conv_geom(8, 16, 1, 1, Hp, Hp, (2, 2)), p1, B, None)
+    a1 = oracle.add(r2, c3)
+    g1 = oracle.gap_pf(a1, 16, a1.shape[1], a1.shape[2], B)
+    return oracle.matmul(oracle.encode(t["Wf"]), g1, t["bf"], "relu").T
+
+
+@pytest.mark.parametrize("B", [4, 32])
+def test_cnn(backend, oracle, tmp_path, B):
+    rng = np.random.default_rng(8 + B)
+    payload, t = cnn_model(rng, B)
+    model = backend.SparseOnnxModel(ow.save(str(tmp_path / "cnn.onnx"), payload))
+    desc = model.describe()
+    assert [d.split()[0] for d in desc] == ["Conv", "MaxPool", "Conv", "Conv", "Add", "GlobalAveragePool", "Gemm"]
+    assert "act=relu" in desc[0] and "act=relu" in desc[2] and "act=none" in desc[3] and "act=relu" in desc[6]
+    X = rng.standard_normal((B, 3, 16, 16)).astype(np.float32)
+    Y = model.run(X)                                                         # C-order NCHW in, (B, 10) out
+    assert Y.shape == (B, 10)
+    assert np.array_equal(Y, oracle_cnn(oracle, t, X))                       # every layer is bit-exact
+    Yt = torch_cnn(t, X)
+    assert rel_err(Y, Yt) <= 1e-5 and np.allclose(Y, Yt, atol=1e-4)
+    assert np.array_equal(model.run(np.asfortranarray(X)), Y)                # any memory order, same answer
+
+
+def test_conv_output_model(backend, oracle, tmp_path):
+    """A graph that ends in a 4-D tensor returns (B, C, H, W) in C order."""
+    from oracle import conv_geom
+    rng = np.random.default_rng(9)
+    W = datagen.he_sparse_conv(rng, 5, 2, 3, .5)
+    payload = ow.model([ow.node("Conv", ["x", "W"], ["y"], kernel_shape=[3, 3], pads=[0, 0, 0, 0])],
+                       [("x", (3, 2, 9, 7))], [("y", (3, 5, 7, 5))], [("W", W)])
+    model = backend.SparseOnnxModel(ow.save(str(tmp_path / "c.onnx"), payload))
+    assert model.output_shape() == [3, 5, 7, 5]
+    X = rng.standard_normal((3, 2, 9, 7)).astype(np.float32)
+    Y = model.run(X)
+    Yo = oracle.conv2d_pf(oracle.encode(W.reshape(5, -1)), conv_geom(2, 5, 3, 3, 9, 7),
+                          np.ascontiguousarray(X.transpose(1, 2, 3, 0)), 3, None)
+    assert Y.shape == (3, 5, 7, 5) and np.array_equal(Y, Yo.transpose(3, 0, 1, 2))
+
+
+def test_matmul_add_bias_folding(backend, oracle, tmp_path):
+    """MatMul followed by Add of a constant vector (how nn.Linear is exported for
+    inputs of rank > 2) becomes the FC layer's bias."""
+    rng = np.random.default_rng(10)
+    W = datagen.magnitude_prune(rng.standard_normal((12, 20)).astype(np.float32), .6)
+    b = rng.standard_normal(12).astype(np.float32)
+    nodes = [ow.node("MatMul", ["x", "Wt"], ["mm"]), ow.node("Add", ["mm", "b"], ["z"]), ow.node("Relu", ["z"], ["y"])]
+    payload = ow.model(nodes, [("x", (6, 20))], [("y", (6, 12))], [("Wt", np.ascontiguousarray(W.T)), ("b", b)])
+    model = backend.SparseOnnxModel(ow.save(str(tmp_path / "f.onnx"), payload))
+    assert len(model.describe()) == 1 and "bias=1" in model.describe()[0] and "act=relu" in model.describe()[0]
+    X = rng.standard_normal((6, 20)).astype(np.float32)
+    assert np.array_equal(model.run(X), oracle.matmul(oracle.encode(W), np.ascontiguousarray(X.T), b, "relu").T)
