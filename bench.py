@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Benchmark of the ELLPACK compute path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+
+Headline workload ("step" = one ellpack_matmul launch over the whole dense block):
+the large FC configuration, W 4096 x 4096 fp32 N(0, 0.02) with per-row top-10 %
+magnitude pruning (uniform r = 410), X 4096 x 256 fp32 N(0,1), bias N(0, 0.1),
+operands resident in HBM.  Prints ONE JSON line: nnz-GFLOP/s as `value`, the HBM
+roofline of the kernel (algorithmic bytes per launch / HIP-event time), the fp32
+VALU fraction, and the same configuration timed on the host cores with the
+reference's own kernel (`oracle/_ref`, kind "reference") or, where that cannot run,
+the plain-C restatement (kind "port").  `extras` holds the other configurations:
+matvec 16384 x 16384 (uniform and Zipf-skewed rows) and the sparse MLP's samples/s.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (os.path.join(ROOT, "sparse-ops_amd"), os.path.join(ROOT, "sparse-ops_amd", "python")):
+    sys.path.insert(0, _p)
+
+import numpy as np  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+VALU_FP32_PEAK_TF = 157.3    # MI355X vector fp32 (packed FMA); 78.6 with plain v_fma_f32
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def alg_bytes(nnz, m, n, C):
+    """Compulsory HBM traffic of one launch, every operand once: Wd + idx over the
+    stored nonzeros, nnz[], bias, X, Y."""
+    return 8 * nnz + 4 * m + 4 * m + 4 * n * C + 4 * m * C
+
+
+def time_launches(ctx, fn, steps, warmup):
+    """-> (wall seconds for `steps` launches, HIP-event ms per launch)."""
+    for _ in range(warmup):
+        fn()
+    ctx.sync()
+    t0 = time.perf_counter()
+    ctx.timer_begin()
+    for _ in range(steps):
+        fn()
+    ev_ms = ctx.timer_end()           # waits for the last launch
+    ctx.sync()
+    wall = time.perf_counter() - t0
+    return wall, ev_ms / steps
+
+
+def cpu_baseline_matmul(E, X, bias, y_gpu, budget_s=15.0):
+    """The same matmul on the host cores: the reference's compiled kernel when it
+    can run here, else the plain-C restatement.  1 warm-up, then the median of as
+    many runs as fit the budget (at least 5, at most 50) -- the reference
+    benchmark's protocol (benchmark-mkl/matmul/bench_matmul.cpp:97-116)."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    from oracle import EllpackArrays, Oracle, Ref
+    cores = len(os.sched_getaffinity(0))
+    threads = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
+    os.environ["OMP_NUM_THREADS"] = str(threads)
+    Eo = EllpackArrays(E.m, E.n, E.r, E.Wd, E.idx, E.nnz)
+    if Ref.available():
+        ref = Ref()
+        h = ref.from_arrays(Eo)
+        Y = np.empty((E.m, X.shape[1]), dtype=np.float32)
+        run, kind = (lambda: ref.matmul(h, X, bias, out=Y)), "reference"
+    else:
+        orc = Oracle()
+        orc.set_num_threads(threads)
+        holder = {}
+        def run():
+            holder["Y"] = orc.matmul(Eo, X, bias)
+        kind = "port"
+    run()
+    times, t_start = [], time.perf_counter()
+    while len(times) < 5 or (len(times) < 50 and time.perf_counter() - t_start < budget_s):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    Ycpu = Y if kind == "reference" else holder["Y"]
+    med = statistics.median(times)
+    flops = 2.0 * E.total_nnz * X.shape[1]
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {
+        "value": round(flops / med / 1e9, 2), "unit": "nnz-GFLOP/s", "cores": threads, "kind": kind,
+        "sample": "same 4096x4096 r=410 C=256 matmul, 1 warm-up + median of %d runs (%.2f ms each)" % (len(times), med * 1e3),
+        "ms_per_step": round(med * 1e3, 4), "cpu_model": model,
+        "gpu_bit_exact_vs_cpu": bool(np.array_equal(Ycpu, y_gpu)),
+        "gpu_max_rel_err_vs_cpu": float(np.abs(Ycpu.astype(np.float64) - y_gpu).max() / np.abs(Ycpu).max()),
+    }
+
+
+def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup):
+    E, x, b = gen()
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, layouts)
+    dx, dB, dy = ctx.array(x), ctx.array(b), ctx.empty((E.m,))
+    _, ms = time_launches(ctx, lambda: ctx.matvec(dE, dx, dB, dy, layout), steps, warmup)
+    nbytes = 8 * E.total_nnz + 4 * E.m + 4 * E.m + 4 * E.n + 4 * E.m
+    out = {"workload": name, "m": E.m, "n": E.n, "r": E.r, "nnz": E.total_nnz, "us_per_launch": round(ms * 1e3, 2),
+           "alg_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1), "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+           "padded_bytes": 8 * E.m * E.r}
+    dE.free()
+    for a in (dx, dB, dy):
+        a.free()
+    return out
+
+
+def bench_mlp(steps, warmup):
+    import datagen
+    import onnx_wire as ow
+    import sparseops_backend as sb
+    Ws = datagen.config4_weights()
+    X = datagen.config4_input()
+    with tempfile.TemporaryDirectory() as d:
+        model = sb.SparseOnnxModel(ow.save(os.path.join(d, "mlp.onnx"), ow.mlp_model(Ws, ["Relu", "Sigmoid", "Tanh", None], 256)))
+    Xf = np.asfortranarray(X)
+    for _ in range(warmup):
+        model.run(Xf)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        model.run(Xf)                       # includes H2D of the input and D2H of the output
+    dt = (time.perf_counter() - t0) / steps
+    dev_ms = model.time_device(steps, warmup)   # chain only, activations resident in HBM
+    return {"workload": "MLP 784-4096-4096-4096-10, 90% sparse, B=256", "layers": model.describe(),
+            "samples_per_s_device_resident": round(256 / (dev_ms * 1e-3), 1), "us_per_batch_device_resident": round(dev_ms * 1e3, 2),
+            "samples_per_s_host_to_host": round(256 / dt, 1), "us_per_batch_host_to_host": round(dt * 1e6, 2),
+            "nnz_gflops_device_resident": round(model.nnz_flops_per_sample() * 256 / (dev_ms * 1e-3) / 1e9, 1)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-extras", action="store_true", help="skip matvec and MLP measurements")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the path shards over the dense-column axis "
+                 "with no exchange; see DESIGN.md); run with --gpus 1")
+
+    import datagen
+    import hipabi
+    ctx = hipabi.Context(0)
+    dev_name, cus = ctx.info()
+    log("device:", dev_name, cus, "CUs")
+
+    E, X, bias = datagen.config3()
+    C = X.shape[1]
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+    dX, dB, dY = ctx.array(X), ctx.array(bias), ctx.empty((E.m, C))
+    step = lambda: ctx.matmul(dE, dX, C, dB, dY, "none")
+    wall, ev_ms = time_launches(ctx, step, args.steps, args.warmup)
+    y_gpu = dY.download()
+    ms_per_step = wall / args.steps * 1e3
+    flops = 2.0 * E.total_nnz * C
+    nbytes = alg_bytes(E.total_nnz, E.m, E.n, C)
+    gbps = nbytes / (ev_ms * 1e-3) / 1e9
+    result = {
+        "metric": "ellpack_matmul nnz-GFLOP/s", "value": round(flops / (ms_per_step * 1e-3) / 1e9, 1), "unit": "nnz-GFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "ellpack_matmul large FC: W 4096x4096 N(0,0.02) per-row top-10%% (r=410, nnz=%d), "
+                               "X 4096x256 N(0,1), bias N(0,0.1), seed 45" % E.total_nnz,
+                   "m": E.m, "n": E.n, "r": E.r, "C": C, "sparsity": 0.9, "device": dev_name},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "ellpack_matmul_kernel", "kernel_us": round(ev_ms * 1e3, 2), "alg_bytes_per_launch": nbytes,
+                     "valu_fp32_frac_of_157.3TF": round(flops / (ev_ms * 1e-3) / 1e12 / VALU_FP32_PEAK_TF, 4),
+                     "valu_fp32_frac_of_78.6TF_unpacked": round(flops / (ev_ms * 1e-3) / 1e12 / (VALU_FP32_PEAK_TF / 2), 4),
+                     "binding_bound": "fp32 VALU / L1-L2 gather bandwidth (t_valu 10.9 us unpacked > t_hbm 2.7 us)"},
+    }
+    if not args.no_cpu:
+        log("timing the host-CPU baseline ...")
+        result["cpu_baseline"] = cpu_baseline_matmul(E, X, bias, y_gpu)
+    else:
+        result["cpu_baseline"] = None
+    if not args.no_extras:
+        extras = {}
+        k = max(20, args.steps // 2)
+        log("matvec 16384^2 uniform ...")
+        extras["matvec_uniform"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 16384x16384, 95% Bernoulli",
+                                                datagen.config2a, hipabi.LAYOUT_ROW, hipabi.LAYOUT_ROW, k, args.warmup)
+        log("matvec 16384^2 zipf ...")
+        extras["matvec_zipf"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048",
+                                             datagen.config2b, hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS, hipabi.LAYOUT_BINS,
+                                             k, args.warmup)
+        log("sparse MLP ...")
+        extras["mlp"] = bench_mlp(k, args.warmup)
+        result["extras"] = extras
+    ctx.close()
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -61,6 +61,11 @@ public:
     std::size_t input_features() const;
     std::size_t output_features() const;
 
+    /// Average milliseconds of one pass of the layer chain over the arena (input
+    /// and output stay in HBM), measured with HIP events on the context's stream
+    /// over `steps` back-to-back passes after `warmup` untimed ones.
+    double time_device(int steps, int warmup) const;
+
     /// One line per executed layer, e.g. "MatMul 4096x784 r=109 act=relu bias=0".
     std::vector<std::string> describe() const;
     /// Sum over sparse layers of 2 * stored nonzeros * output columns per sample.

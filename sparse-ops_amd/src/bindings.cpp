@@ -201,6 +201,7 @@ PYBIND11_MODULE(sparseops_backend, mod)
         .def("output_shape", &SparseOnnxModel::output_shape)
         .def("input_shape", &SparseOnnxModel::input_shape)
         .def("batch", &SparseOnnxModel::batch)
+        .def("time_device", &SparseOnnxModel::time_device, py::arg("steps"), py::arg("warmup") = 3)
         .def("describe", &SparseOnnxModel::describe)
         .def("nnz_flops_per_sample", &SparseOnnxModel::nnz_flops_per_sample);
 }

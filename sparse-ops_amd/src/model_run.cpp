@@ -115,3 +115,17 @@ void SparseOnnxModel::run_device(const float *dInput, uint32_t B, float *dOutput
     }
     M.enqueue_layers(dInput, dOutput);
 }
+
+double SparseOnnxModel::time_device(int steps, int warmup) const
+{
+    Impl &M = *impl_;
+    if (steps <= 0) throw std::runtime_error("time_device: steps must be positive");
+    so_ctx *ctx = context();
+    std::lock_guard<std::mutex> lock(context_mutex());
+    for (int i = 0; i < warmup; ++i) M.launch_chain();
+    check(so_timer_begin(ctx), "so_timer_begin");
+    for (int i = 0; i < steps; ++i) M.launch_chain();
+    float ms = 0.0f;
+    check(so_timer_end(ctx, &ms), "so_timer_end");
+    return double(ms) / steps;
+}
