@@ -150,6 +150,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extras", action="store_true", help="skip matvec and MLP measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch a plain 256 MiB copy kernel (scale factor for rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path shards over the dense-column axis "
@@ -186,6 +188,18 @@ def main():
                      "valu_fp32_frac_of_78.6TF_unpacked": round(flops / (ev_ms * 1e-3) / 1e12 / (VALU_FP32_PEAK_TF / 2), 4),
                      "binding_bound": "fp32 VALU / L1-L2 gather bandwidth (t_valu 10.9 us unpacked > t_hbm 2.7 us)"},
     }
+    if args.calibrate_copy:
+        # A plain copy of known size (act_kernel<NONE>: reads N floats, writes N floats)
+        # so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings can be scaled.
+        n_cal = 64 * 1024 * 1024
+        src, dst = ctx.empty((n_cal,)), ctx.empty((n_cal,))
+        ctx.fill_zero(src)
+        for _ in range(5):
+            ctx.act("none", src, n_cal, dst)
+        ctx.sync()
+        result["calibration_copy"] = {"kernel": "act_kernel<0>", "bytes_read": 4 * n_cal, "bytes_written": 4 * n_cal}
+        src.free()
+        dst.free()
     if not args.no_cpu:
         log("timing the host-CPU baseline ...")
         result["cpu_baseline"] = cpu_baseline_matmul(E, X, bias, y_gpu)

@@ -13,6 +13,8 @@
 // its own tiles' slice of X.
 #include "so_internal.h"
 
+#include <cstdlib>
+
 namespace {
 
 constexpr int kWavesPerGroup = 4;
@@ -96,21 +98,36 @@ void ellpack_matmul_kernel(const float *__restrict__ Wd, const uint32_t *__restr
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = b;
 
-    uint32_t j = 0;
-    for (; j + kUnroll <= cnt; j += kUnroll) {
-        float w[kUnroll];
-        float x[kUnroll][VEC];
+    // Batches of kUnroll nonzeros, double-buffered in registers: the gathers of
+    // batch b+1 are issued before batch b is consumed, so a wave always has one
+    // batch of loads in flight while it waits for scalar loads or does FMAs.
+    // The FMAs themselves stay strictly in slot order.
+    float wa[kUnroll], wb[kUnroll];
+    float xa[kUnroll][VEC], xb[kUnroll][VEC];
+    auto issue = [&](uint32_t j0, float (&w)[kUnroll], float (&x)[kUnroll][VEC]) {
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            w[u] = wrow[j + u];
-            load_vec<VEC>(xcol + (size_t)irow[j + u] * C, x[u]);
+            w[u] = wrow[j0 + u];
+            load_vec<VEC>(xcol + (size_t)irow[j0 + u] * C, x[u]);
         }
+    };
+    auto consume = [&](const float (&w)[kUnroll], const float (&x)[kUnroll][VEC]) {
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
 #pragma unroll
             for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(w[u], x[u][v], acc[v]);
+    };
+    const uint32_t nb = cnt / kUnroll;
+    if (nb) issue(0, wa, xa);
+    uint32_t bi = 0;
+    for (; bi + 1 < nb; bi += 2) {
+        issue((bi + 1) * kUnroll, wb, xb);
+        consume(wa, xa);
+        if (bi + 2 < nb) issue((bi + 2) * kUnroll, wa, xa);
+        consume(wb, xb);
     }
-    for (; j < cnt; ++j) {
+    if (nb & 1u) consume(wa, xa);
+    for (uint32_t j = nb * kUnroll; j < cnt; ++j) {
         const float w = wrow[j];
         float x[VEC];
         load_vec<VEC>(xcol + (size_t)irow[j] * C, x);
@@ -169,6 +186,10 @@ extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX
     int vec = 1;
     if (C % 256 == 0 && (align & 15) == 0) vec = 4;
     else if (C % 128 == 0 && (align & 7) == 0) vec = 2;
+    if (const char *e = getenv("SPARSEOPS_MATMUL_VEC")) {   // tuning override: narrower lanes only
+        const int v = atoi(e);
+        if ((v == 1 || v == 2) && v < vec) vec = v;
+    }
     if (vec == 4) launch_act<4>(ctx, E, dX, C, dBias, dY, act);
     else if (vec == 2) launch_act<2>(ctx, E, dX, C, dBias, dY, act);
     else launch_act<1>(ctx, E, dX, C, dBias, dY, act);
