@@ -194,3 +194,26 @@ def test_matmul_add_bias_folding(backend, oracle, tmp_path):
     assert len(model.describe()) == 1 and "bias=1" in model.describe()[0] and "act=relu" in model.describe()[0]
     X = rng.standard_normal((6, 20)).astype(np.float32)
     assert np.array_equal(model.run(X), oracle.matmul(oracle.encode(W), np.ascontiguousarray(X.T), b, "relu").T)
+
+
+def test_python_runtime_wrappers(oracle, tmp_path):
+    """python/cpp_backend.py and python/sparse_onnx.py (the reference's python/ package)."""
+    from python.cpp_backend import encode, matmul, matvec
+    from python.sparse_onnx import OnnxSparseModel
+    rng = np.random.default_rng(13)
+    Ws = [datagen.magnitude_prune(rng.standard_normal((24, 16)).astype(np.float32), .6),
+          datagen.magnitude_prune(rng.standard_normal((8, 24)).astype(np.float32), .6)]
+    bs = [rng.standard_normal(24).astype(np.float32), rng.standard_normal(8).astype(np.float32)]
+    path = ow.save(str(tmp_path / "g.onnx"), ow.mlp_model(Ws, ["Relu", None], 4, bs, use_gemm=True))
+    model = OnnxSparseModel(path)
+    x = rng.standard_normal(16).astype(np.float32)
+    y = model.run(x)                                          # 1-D input: matvec path
+    ref = Ws[1].astype(np.float64) @ np.maximum(Ws[0].astype(np.float64) @ x + bs[0], 0) + bs[1]
+    assert y.shape == (8,) and rel_err(y, ref) <= 1e-5
+    X = rng.standard_normal((16, 5)).astype(np.float32)       # (n, C) input: matmul path
+    Y = model.run(X)
+    H = oracle.matmul(oracle.encode(Ws[0]), X, bs[0], "relu")
+    assert np.array_equal(Y, oracle.matmul(oracle.encode(Ws[1]), H, bs[1]))
+    E = encode(Ws[0])
+    assert np.array_equal(matmul(E, X, bs[0]), oracle.matmul(oracle.encode(Ws[0]), X, bs[0]))
+    assert rel_err(matvec(E, x, bs[0]), Ws[0].astype(np.float64) @ x + bs[0]) <= 1e-5
