@@ -143,6 +143,21 @@ def bench_mlp(steps, warmup):
             "nnz_gflops_device_resident": round(model.nnz_flops_per_sample() * 256 / (dev_ms * 1e-3) / 1e9, 1)}
 
 
+def bench_cnn(steps, warmup):
+    import datagen
+    import onnx_wire as ow
+    import sparseops_backend as sb
+    payload, _ = datagen.resnet18_onnx(seed=47, batch=32, hw=224, sparsity=0.8)
+    with tempfile.TemporaryDirectory() as d:
+        model = sb.SparseOnnxModel(ow.save(os.path.join(d, "r18.onnx"), payload))
+    dev_ms = model.time_device(steps, warmup)
+    flops = model.nnz_flops_per_sample() * 32
+    return {"workload": "ResNet-18-shaped conv stack (no BN), 80% sparse, B=32, 3x224x224, implicit im2col",
+            "layers": len(model.describe()), "ms_per_batch_device_resident": round(dev_ms, 3),
+            "samples_per_s_device_resident": round(32 / (dev_ms * 1e-3), 1),
+            "nnz_gflop_per_batch": round(flops / 1e9, 2), "nnz_gflops": round(flops / (dev_ms * 1e-3) / 1e9, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -217,6 +232,8 @@ def main():
                                              k, args.warmup)
         log("sparse MLP ...")
         extras["mlp"] = bench_mlp(k, args.warmup)
+        log("sparse CNN ...")
+        extras["cnn"] = bench_cnn(max(5, args.steps // 20), 2)
         result["extras"] = extras
     ctx.close()
     print(json.dumps(result), flush=True)

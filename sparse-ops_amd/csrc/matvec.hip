@@ -3,16 +3,18 @@
 // The product is a pure stream of the stored (weight, column) pairs -- 8 bytes
 // per nonzero and one multiply-add -- so the kernels are built around HBM
 // bandwidth: x is staged once per workgroup in LDS when it fits (the gathers
-// then never leave the CU), the pairs are read with 16-byte loads, and only the
-// first nnz[i] slots of a row are touched, so ELLPACK padding is never streamed.
+// then never leave the CU), the pairs are read with 16-byte non-temporal loads,
+// four per lane in flight, and only the first nnz[i] slots of a row are touched,
+// so ELLPACK padding is never streamed.
 //
-//   wave kernel   one wavefront per row on the row-major arrays; lanes take
-//                 aligned groups of four slots, partial sums are combined with a
-//                 butterfly of lane exchanges.
-//   group kernel  4 or 16 lanes per row, for the short-row classes of a binned
-//                 upload (skewed matrices).
-//   slot kernel   one lane per row on the slot-major arrays (consecutive rows'
-//                 k-th nonzeros are contiguous, so loads coalesce across lanes).
+//   rows kernel    one wavefront per row on the row-major arrays; lanes take
+//                  aligned groups of four slots, partial sums are combined with a
+//                  butterfly of lane exchanges.
+//   binned kernel  one launch over three length classes (skewed matrices): whole
+//                  waves for long rows, 16 or 4 lanes per row for short ones;
+//                  workgroups of the long class are dispatched first.
+//   slot kernel    one lane per row on the slot-major arrays (consecutive rows'
+//                  k-th nonzeros are contiguous, so loads coalesce across lanes).
 //
 // Reference: ellpack_matvec, src/ellpack_matvec.cpp:20-147.  The reference sums
 // 16 interleaved partials and a tree (:72-96); the orders here differ, so results
@@ -23,7 +25,8 @@
 
 namespace {
 
-constexpr int kBlock = 512;
+constexpr int kBlock = 1024;
+constexpr int kWavesPerBlock = kBlock / 64;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -46,67 +49,114 @@ __device__ __forceinline__ const float *stage_x(const float *__restrict__ x, uin
     return lds;
 }
 
+// Dot product of one row with x, computed by a whole wave.  The row's slots
+// [beg, end) are covered by aligned groups of four; a lane loads up to four such
+// groups before using any (addresses past the row are clamped onto its last
+// group and every slot outside [beg, end) is masked to an exact no-op).
+__device__ __forceinline__ float wave_row_dot(const f32x4 *__restrict__ Wd4, const u32x4 *__restrict__ idx4,
+                                              uint64_t beg, uint64_t end, const float *xs, uint32_t lane)
+{
+    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+    if (end == beg) return 0.0f;
+    const uint64_t qlast = (end - 1) >> 2;
+    for (uint64_t q0 = (beg >> 2) + lane; q0 <= qlast; q0 += 256) {
+        f32x4 w[4];
+        u32x4 c[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint64_t q = std::min<uint64_t>(q0 + 64u * u, qlast);
+            w[u] = __builtin_nontemporal_load(Wd4 + q);
+            c[u] = __builtin_nontemporal_load(idx4 + q);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint64_t e = (q0 + 64u * u) << 2;
+            const bool v0 = e >= beg && e < end, v1 = e + 1 >= beg && e + 1 < end;
+            const bool v2 = e + 2 >= beg && e + 2 < end, v3 = e + 3 >= beg && e + 3 < end;
+            const float x0 = xs[v0 ? c[u].x : 0u], x1 = xs[v1 ? c[u].y : 0u];
+            const float x2 = xs[v2 ? c[u].z : 0u], x3 = xs[v3 ? c[u].w : 0u];
+            a0 = __builtin_fmaf(v0 ? w[u].x : 0.0f, v0 ? x0 : 0.0f, a0);
+            a1 = __builtin_fmaf(v1 ? w[u].y : 0.0f, v1 ? x1 : 0.0f, a1);
+            a2 = __builtin_fmaf(v2 ? w[u].z : 0.0f, v2 ? x2 : 0.0f, a2);
+            a3 = __builtin_fmaf(v3 ? w[u].w : 0.0f, v3 ? x3 : 0.0f, a3);
+        }
+    }
+    return group_sum<64>((a0 + a1) + (a2 + a3));
+}
+
+template <int G>
+__device__ __forceinline__ float group_row_dot(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
+                                               uint64_t base, uint32_t cnt, const float *xs, uint32_t sub)
+{
+    float a = 0.0f;
+    for (uint32_t j = sub; j < cnt; j += G) a = __builtin_fmaf(Wd[base + j], xs[idx[base + j]], a);
+    return group_sum<G>(a);
+}
+
 // rows == nullptr: row ids are 0..count-1; otherwise the ids come from the list.
 template <bool XLDS>
 __global__ __launch_bounds__(kBlock)
-void matvec_wave_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
-                        const uint32_t *__restrict__ nnz, const uint32_t *__restrict__ rows,
-                        uint32_t count, uint32_t r, const float *__restrict__ x, uint32_t n,
+void matvec_rows_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
+                        const uint32_t *__restrict__ nnz, uint32_t count, uint32_t r,
+                        const float *__restrict__ x, uint32_t n,
                         const float *__restrict__ bias, float *__restrict__ y)
 {
     extern __shared__ float lds_x[];
     const float *xs = stage_x<XLDS>(x, n, lds_x);
     const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wave = (blockIdx.x * kBlock + threadIdx.x) >> 6;
-    const uint32_t nwaves = (gridDim.x * kBlock) >> 6;
-
-    for (uint32_t g = wave; g < count; g += nwaves) {
-        const uint32_t row = rows ? rows[g] : g;
+    const uint32_t wave = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    const uint32_t nwaves = gridDim.x * kWavesPerBlock;
+    for (uint32_t row = wave; row < count; row += nwaves) {
         const uint64_t beg = (uint64_t)row * r;
-        const uint64_t end = beg + nnz[row];
-        float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
-        // Aligned groups of four slots covering [beg, end); slots of neighbouring
-        // rows that share the first or last group are masked out.
-        for (uint64_t q = (beg >> 2) + lane; (q << 2) < end; q += 64) {
-            const f32x4 w = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(Wd) + q);
-            const u32x4 c = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(idx) + q);
-            const uint64_t e = q << 2;
-            const bool v0 = e >= beg && e < end, v1 = e + 1 >= beg && e + 1 < end;
-            const bool v2 = e + 2 >= beg && e + 2 < end, v3 = e + 3 >= beg && e + 3 < end;
-            const float x0 = v0 ? xs[c.x] : 0.0f, x1 = v1 ? xs[c.y] : 0.0f;
-            const float x2 = v2 ? xs[c.z] : 0.0f, x3 = v3 ? xs[c.w] : 0.0f;
-            a0 = __builtin_fmaf(v0 ? w.x : 0.0f, x0, a0);
-            a1 = __builtin_fmaf(v1 ? w.y : 0.0f, x1, a1);
-            a2 = __builtin_fmaf(v2 ? w.z : 0.0f, x2, a2);
-            a3 = __builtin_fmaf(v3 ? w.w : 0.0f, x3, a3);
-        }
-        const float s = group_sum<64>((a0 + a1) + (a2 + a3));
+        const float s = wave_row_dot(reinterpret_cast<const f32x4 *>(Wd), reinterpret_cast<const u32x4 *>(idx),
+                                     beg, beg + nnz[row], xs, lane);
         if (lane == 0) y[row] = (bias ? bias[row] : 0.0f) + s;
     }
 }
 
-template <int G, bool XLDS>
+struct BinArgs {
+    const uint32_t *rows64, *rows16, *rows4;   // row ids per length class
+    uint32_t n64, n16, n4;                     // rows per class
+    uint32_t b64, b16;                         // workgroups given to the 64- and 16-lane classes
+};
+
+template <bool XLDS>
 __global__ __launch_bounds__(kBlock)
-void matvec_group_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
-                         const uint32_t *__restrict__ nnz, const uint32_t *__restrict__ rows,
-                         uint32_t count, uint32_t r, const float *__restrict__ x, uint32_t n,
-                         const float *__restrict__ bias, float *__restrict__ y)
+void matvec_binned_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
+                          const uint32_t *__restrict__ nnz, BinArgs ba, uint32_t r,
+                          const float *__restrict__ x, uint32_t n,
+                          const float *__restrict__ bias, float *__restrict__ y)
 {
     extern __shared__ float lds_x[];
     const float *xs = stage_x<XLDS>(x, n, lds_x);
-    const uint32_t sub = threadIdx.x % G;
-    const uint32_t group = (blockIdx.x * kBlock + threadIdx.x) / G;
-    const uint32_t ngroups = (gridDim.x * kBlock) / G;
-
-    for (uint32_t g = group; g < count; g += ngroups) {
-        const uint32_t row = rows ? rows[g] : g;
-        const uint64_t base = (uint64_t)row * r;
-        const uint32_t cnt = nnz[row];
-        float a = 0.0f;
-        for (uint32_t j = sub; j < cnt; j += G)
-            a = __builtin_fmaf(Wd[base + j], xs[idx[base + j]], a);
-        a = group_sum<G>(a);
-        if (sub == 0) y[row] = (bias ? bias[row] : 0.0f) + a;
+    const uint32_t b = blockIdx.x;
+    if (b < ba.b64) {
+        const uint32_t lane = threadIdx.x & 63u;
+        const uint32_t stride = ba.b64 * kWavesPerBlock;
+        for (uint32_t g = b * kWavesPerBlock + (threadIdx.x >> 6); g < ba.n64; g += stride) {
+            const uint32_t row = ba.rows64[g];
+            const uint64_t beg = (uint64_t)row * r;
+            const float s = wave_row_dot(reinterpret_cast<const f32x4 *>(Wd), reinterpret_cast<const u32x4 *>(idx),
+                                         beg, beg + nnz[row], xs, lane);
+            if (lane == 0) y[row] = (bias ? bias[row] : 0.0f) + s;
+        }
+    } else if (b < ba.b64 + ba.b16) {
+        const uint32_t sub = threadIdx.x & 15u;
+        const uint32_t stride = ba.b16 * (kBlock / 16);
+        for (uint32_t g = (b - ba.b64) * (kBlock / 16) + (threadIdx.x >> 4); g < ba.n16; g += stride) {
+            const uint32_t row = ba.rows16[g];
+            const float s = group_row_dot<16>(Wd, idx, (uint64_t)row * r, nnz[row], xs, sub);
+            if (sub == 0) y[row] = (bias ? bias[row] : 0.0f) + s;
+        }
+    } else {
+        const uint32_t sub = threadIdx.x & 3u;
+        const uint32_t b4 = gridDim.x - ba.b64 - ba.b16;
+        const uint32_t stride = b4 * (kBlock / 4);
+        for (uint32_t g = (b - ba.b64 - ba.b16) * (kBlock / 4) + (threadIdx.x >> 2); g < ba.n4; g += stride) {
+            const uint32_t row = ba.rows4[g];
+            const float s = group_row_dot<4>(Wd, idx, (uint64_t)row * r, nnz[row], xs, sub);
+            if (sub == 0) y[row] = (bias ? bias[row] : 0.0f) + s;
+        }
     }
 }
 
@@ -131,51 +181,29 @@ void matvec_slot_kernel(const float *__restrict__ WdT, const uint32_t *__restric
     }
 }
 
-// Workgroups to launch for `work` row-units when one workgroup handles `per` of
-// them per pass: enough to cover the work, at most a few per compute unit (each
-// workgroup re-stages x, so more than that only adds traffic).
-uint32_t grid_for(const so_ctx *ctx, uint64_t work, uint32_t per, bool xlds)
-{
-    const uint32_t need = so_ceil_div(work, per);
-    const uint32_t cap = (uint32_t)ctx->compute_units * (xlds ? 2u : 8u);
-    return std::max(1u, std::min(need, cap));
-}
-
-bool enable_lds(const void *kernel, size_t bytes)
-{
-    if (bytes <= 48 * 1024) return true;
-    return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) == hipSuccess;
-}
-
-template <typename K, typename... Args>
-so_status launch_x(so_ctx *ctx, K k_lds, K k_gl, uint64_t work, uint32_t per, uint32_t n, Args... args)
+// LDS staging of x is worth its per-workgroup copy only when a workgroup then
+// serves many nonzeros from it; it needs n floats of LDS (set up once per kernel).
+template <typename K>
+bool use_lds(const so_ctx *ctx, K kernel, uint32_t n, uint64_t nnz_total, uint32_t blocks)
 {
     const size_t lds = (size_t)n * sizeof(float);
-    // x in LDS pays when each workgroup handles many rows; for a handful of rows
-    // the staging copy would dominate.
-    bool xlds = lds > 0 && lds <= (size_t)ctx->max_lds_bytes && work >= 4ull * per &&
-                enable_lds((const void *)k_lds, lds);
-    if (!xlds) (void)hipGetLastError();
-    const uint32_t blocks = grid_for(ctx, work, per, xlds);
-    if (xlds) k_lds<<<blocks, kBlock, lds, ctx->stream>>>(args...);
-    else k_gl<<<blocks, kBlock, 0, ctx->stream>>>(args...);
-    SO_LAUNCH_CHECK();
-    return SO_OK;
-}
-
-so_status run_wave(so_ctx *ctx, const so_ellpack *E, const uint32_t *rows, uint32_t count,
-                   const float *dx, const float *dBias, float *dy)
-{
-    return launch_x(ctx, matvec_wave_kernel<true>, matvec_wave_kernel<false>, count, kBlock / 64, E->n,
-                    E->d_Wd, E->d_idx, E->d_nnz, rows, count, E->r, dx, E->n, dBias, dy);
-}
-
-template <int G>
-so_status run_group(so_ctx *ctx, const so_ellpack *E, const uint32_t *rows, uint32_t count,
-                    const float *dx, const float *dBias, float *dy)
-{
-    return launch_x(ctx, matvec_group_kernel<G, true>, matvec_group_kernel<G, false>, count, kBlock / G,
-                    E->n, E->d_Wd, E->d_idx, E->d_nnz, rows, count, E->r, dx, E->n, dBias, dy);
+    if (lds == 0 || lds > (size_t)ctx->max_lds_bytes) return false;
+    if (nnz_total < (uint64_t)n * blocks) return false;   // fewer gathers than staged elements
+    if (lds > 48 * 1024) {
+        static thread_local const void *configured[8] = {};
+        const void *k = (const void *)kernel;
+        bool done = false;
+        for (const void *c : configured) done |= (c == k);
+        if (!done) {
+            if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, ctx->max_lds_bytes) != hipSuccess) {
+                (void)hipGetLastError();
+                return false;
+            }
+            for (const void *&c : configured)
+                if (!c) { c = k; break; }
+        }
+    }
+    return true;
 }
 
 } // namespace
@@ -196,18 +224,43 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
                "so_matvec: unknown layout %d", layout);
     SO_REQUIRE((E->layouts & layout) != 0, "so_matvec: layout %d was not uploaded", layout);
 
-    if (layout == SO_LAYOUT_ROW) return run_wave(ctx, E, nullptr, E->m, dx, dBias, dy);
-    if (layout == SO_LAYOUT_SLOT)
-        return launch_x(ctx, matvec_slot_kernel<true>, matvec_slot_kernel<false>, E->m, kBlock, E->n,
-                        E->d_WdT, E->d_idxT, E->d_nnz, E->m, dx, E->n, dBias, dy);
-    // Binned: one launch per non-empty length class; every row is in exactly one.
-    for (const so_bin &b : E->bins) {
-        if (b.count == 0) continue;
-        so_status s;
-        if (b.group == 4) s = run_group<4>(ctx, E, b.d_rows, b.count, dx, dBias, dy);
-        else if (b.group == 16) s = run_group<16>(ctx, E, b.d_rows, b.count, dx, dBias, dy);
-        else s = run_wave(ctx, E, b.d_rows, b.count, dx, dBias, dy);
-        if (s != SO_OK) return s;
+    const uint32_t cus = (uint32_t)ctx->compute_units;
+    const size_t lds = (size_t)E->n * sizeof(float);
+    if (layout == SO_LAYOUT_ROW) {
+        // Two resident workgroups per compute unit: 32 waves streaming per CU.
+        const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, kWavesPerBlock), 2u * cus));
+        if (use_lds(ctx, matvec_rows_kernel<true>, E->n, E->total_nnz, blocks))
+            matvec_rows_kernel<true><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->r,
+                                                                           dx, E->n, dBias, dy);
+        else
+            matvec_rows_kernel<false><<<blocks, kBlock, 0, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->r,
+                                                                          dx, E->n, dBias, dy);
+    } else if (layout == SO_LAYOUT_SLOT) {
+        const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, kBlock), 2u * cus));
+        if (use_lds(ctx, matvec_slot_kernel<true>, E->n, E->total_nnz, blocks))
+            matvec_slot_kernel<true><<<blocks, kBlock, lds, ctx->stream>>>(E->d_WdT, E->d_idxT, E->d_nnz, E->m,
+                                                                           dx, E->n, dBias, dy);
+        else
+            matvec_slot_kernel<false><<<blocks, kBlock, 0, ctx->stream>>>(E->d_WdT, E->d_idxT, E->d_nnz, E->m,
+                                                                          dx, E->n, dBias, dy);
+    } else {
+        // One launch over the three length classes.  bins[] is ordered 4, 16, 64 lanes.
+        BinArgs ba;
+        ba.rows4 = E->bins[0].d_rows;   ba.n4 = E->bins[0].count;
+        ba.rows16 = E->bins[1].d_rows;  ba.n16 = E->bins[1].count;
+        ba.rows64 = E->bins[2].d_rows;  ba.n64 = E->bins[2].count;
+        ba.b64 = std::min(so_ceil_div(ba.n64, kWavesPerBlock), 2u * cus);
+        ba.b16 = std::min(so_ceil_div(ba.n16, kBlock / 16), std::max(1u, cus / 4));
+        const uint32_t b4 = std::min(so_ceil_div(ba.n4, kBlock / 4), std::max(1u, cus / 4));
+        const uint32_t blocks = ba.b64 + ba.b16 + b4;
+        if (blocks == 0) return SO_OK;
+        if (use_lds(ctx, matvec_binned_kernel<true>, E->n, E->total_nnz, blocks))
+            matvec_binned_kernel<true><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, ba, E->r,
+                                                                             dx, E->n, dBias, dy);
+        else
+            matvec_binned_kernel<false><<<blocks, kBlock, 0, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, ba, E->r,
+                                                                            dx, E->n, dBias, dy);
     }
+    SO_LAUNCH_CHECK();
     return SO_OK;
 }

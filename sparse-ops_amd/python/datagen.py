@@ -158,3 +158,45 @@ def he_sparse_conv(rng, cout, cin, k, sparsity=0.8):
     W = rng.standard_normal((cout, cin, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / fan_in))
     W[rng.random(W.shape, dtype=np.float32) < sparsity] = 0.0
     return W
+
+
+def resnet18_onnx(seed=47, batch=32, hw=224, sparsity=0.8, classes=1000, width=64):
+    """ResNet-18-shaped graph without BatchNorm (as a constant-folded export has it,
+    the reference's tests/test_resnet.py:57-70): 7x7/2 stem + 3x3/2 max-pool, four
+    stages of two basic blocks (3x3 convs, 1x1 stride-2 projection on the first skip
+    of stages 2-4), Add + ReLU, global average pool, Flatten, Gemm.  Conv weights
+    He-initialised with i.i.d. Bernoulli sparsity.  Returns (onnx bytes, tensors)."""
+    import onnx_wire as ow
+    rng = np.random.default_rng(seed)
+    t, nodes = {}, []
+
+    def conv(x, name, cin, cout, k, stride, pad, relu):
+        t[name + "_w"] = he_sparse_conv(rng, cout, cin, k, sparsity)
+        t[name + "_b"] = rng.standard_normal(cout, dtype=np.float32) * np.float32(0.01)
+        nodes.append(ow.node("Conv", [x, name + "_w", name + "_b"], [name], kernel_shape=[k, k],
+                             pads=[pad] * 4, strides=[stride, stride], dilations=[1, 1], group=1))
+        if relu:
+            nodes.append(ow.node("Relu", [name], [name + "_r"]))
+            return name + "_r"
+        return name
+
+    x = conv("input", "stem", 3, width, 7, 2, 3, True)
+    nodes.append(ow.node("MaxPool", [x], ["pool"], kernel_shape=[3, 3], strides=[2, 2], pads=[1, 1, 1, 1]))
+    x, cin = "pool", width
+    for s, cout in enumerate((width, 2 * width, 4 * width, 8 * width)):
+        for b in range(2):
+            stride = 2 if (s > 0 and b == 0) else 1
+            nm = "s%db%d" % (s, b)
+            y = conv(x, nm + "c1", cin, cout, 3, stride, 1, True)
+            y = conv(y, nm + "c2", cout, cout, 3, 1, 1, False)
+            skip = x if (stride == 1 and cin == cout) else conv(x, nm + "proj", cin, cout, 1, stride, 0, False)
+            nodes.append(ow.node("Add", [y, skip], [nm + "add"]))
+            nodes.append(ow.node("Relu", [nm + "add"], [nm + "out"]))
+            x, cin = nm + "out", cout
+    nodes.append(ow.node("GlobalAveragePool", [x], ["gap"]))
+    nodes.append(ow.node("Flatten", ["gap"], ["flat"], axis=1))
+    t["fc_w"] = (rng.standard_normal((classes, cin), dtype=np.float32) * np.float32(1.0 / np.sqrt(cin)))
+    t["fc_b"] = rng.standard_normal(classes, dtype=np.float32) * np.float32(0.01)
+    nodes.append(ow.node("Gemm", ["flat", "fc_w", "fc_b"], ["logits"], alpha=1.0, beta=1.0, transB=1))
+    payload = ow.model(nodes, [("input", (batch, 3, hw, hw))], [("logits", (batch, classes))], list(t.items()))
+    return payload, t

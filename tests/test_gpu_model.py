@@ -217,3 +217,38 @@ def test_python_runtime_wrappers(oracle, tmp_path):
     E = encode(Ws[0])
     assert np.array_equal(matmul(E, X, bs[0]), oracle.matmul(oracle.encode(Ws[0]), X, bs[0]))
     assert rel_err(matvec(E, x, bs[0]), Ws[0].astype(np.float64) @ x + bs[0]) <= 1e-5
+
+
+def torch_resnet(t, X, width=64):
+    import torch
+    import torch.nn.functional as F
+    T = {k: torch.from_numpy(v).double() for k, v in t.items()}
+    x = F.relu(F.conv2d(torch.from_numpy(X).double(), T["stem_w"], T["stem_b"], stride=2, padding=3))
+    x = F.max_pool2d(x, 3, 2, 1)
+    cin = width
+    for s, cout in enumerate((width, 2 * width, 4 * width, 8 * width)):
+        for b in range(2):
+            stride = 2 if (s > 0 and b == 0) else 1
+            nm = "s%db%d" % (s, b)
+            y = F.relu(F.conv2d(x, T[nm + "c1_w"], T[nm + "c1_b"], stride=stride, padding=1))
+            y = F.conv2d(y, T[nm + "c2_w"], T[nm + "c2_b"], padding=1)
+            skip = x if (stride == 1 and cin == cout) else F.conv2d(x, T[nm + "proj_w"], T[nm + "proj_b"], stride=stride)
+            x, cin = F.relu(y + skip), cout
+    return (x.mean(dim=(2, 3)) @ T["fc_w"].T + T["fc_b"]).numpy()
+
+
+def test_resnet18_shaped(backend, oracle, tmp_path):
+    """Config 5 topology at reduced size (B=4, 64x64, width 32) against the oracle
+    chain (bit-exact) and torch fp64 (1e-5 relative, the reference's atol=1e-4)."""
+    from graph_oracle import run_graph
+    payload, t = datagen.resnet18_onnx(seed=47, batch=4, hw=64, sparsity=0.8, classes=100, width=32)
+    model = backend.SparseOnnxModel(ow.save(str(tmp_path / "r18.onnx"), payload))
+    desc = model.describe()
+    assert sum(d.startswith("Conv") for d in desc) == 20 and sum(d.startswith("Add") for d in desc) == 8
+    assert model.output_shape() == [4, 100]
+    X = np.random.default_rng(1).standard_normal((4, 3, 64, 64)).astype(np.float32)
+    Y = model.run(X)
+    Yo = run_graph(oracle, payload, X)
+    assert np.array_equal(Y, Yo)
+    Yt = torch_resnet(t, X, width=32)
+    assert rel_err(Y, Yt) <= 1e-5 and np.allclose(Y, Yt, atol=1e-4)
