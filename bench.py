@@ -29,6 +29,10 @@ import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 VALU_FP32_PEAK_TF = 157.3    # MI355X vector fp32 (packed FMA); 78.6 with plain v_fma_f32
+# HBM-side bytes per launch of the headline kernel, from two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE) scaled by a plain copy of known size; see the pmc summary
+# under profiles/.  None until measured for the kernel that currently runs.
+MEASURED_TRAFFIC_BYTES = 91_300_000   # ellpack_matmul_tiled_kernel: 87.1 MB fetched + 4.19 MB written
 
 
 def log(*a):
@@ -180,11 +184,18 @@ def main():
 
     E, X, bias = datagen.config3()
     C = X.shape[1]
-    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+    # ROW is the encoder's layout; TILED adds the K-tiled copy that so_matmul's
+    # LDS-staged kernel consumes (same nonzeros, same order inside every row).
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, hipabi.LAYOUT_ROW | hipabi.LAYOUT_TILED)
     dX, dB, dY = ctx.array(X), ctx.array(bias), ctx.empty((E.m, C))
     step = lambda: ctx.matmul(dE, dX, C, dB, dY, "none")
     wall, ev_ms = time_launches(ctx, step, args.steps, args.warmup)
     y_gpu = dY.download()
+    # the row-per-wave kernel on the plain ROW layout, for comparison
+    dE_row = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, hipabi.LAYOUT_ROW)
+    _, ev_ms_row = time_launches(ctx, lambda: ctx.matmul(dE_row, dX, C, dB, dY, "none"), max(20, args.steps // 4), 5)
+    row_bits_equal = bool(np.array_equal(dY.download(), y_gpu))
+    dE_row.free()
     ms_per_step = wall / args.steps * 1e3
     flops = 2.0 * E.total_nnz * C
     nbytes = alg_bytes(E.total_nnz, E.m, E.n, C)
@@ -197,8 +208,9 @@ def main():
                                "X 4096x256 N(0,1), bias N(0,0.1), seed 45" % E.total_nnz,
                    "m": E.m, "n": E.n, "r": E.r, "C": C, "sparsity": 0.9, "device": dev_name},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "ellpack_matmul_kernel", "kernel_us": round(ev_ms * 1e3, 2), "alg_bytes_per_launch": nbytes,
+                     "frac": round(gbps / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel": "ellpack_matmul_tiled_kernel", "kernel_us": round(ev_ms * 1e3, 2), "alg_bytes_per_launch": nbytes,
+                     "row_kernel_us": round(ev_ms_row * 1e3, 2), "row_kernel_same_bits": row_bits_equal,
                      "valu_fp32_frac_of_157.3TF": round(flops / (ev_ms * 1e-3) / 1e12 / VALU_FP32_PEAK_TF, 4),
                      "valu_fp32_frac_of_78.6TF_unpacked": round(flops / (ev_ms * 1e-3) / 1e12 / (VALU_FP32_PEAK_TF / 2), 4),
                      "binding_bound": "fp32 VALU / L1-L2 gather bandwidth (t_valu 10.9 us unpacked > t_hbm 2.7 us)"},

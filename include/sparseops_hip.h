@@ -58,8 +58,13 @@ enum { SO_ACT_NONE = 0, SO_ACT_RELU = 1, SO_ACT_SIGMOID = 2, SO_ACT_TANH = 3 };
  *        nonzeros of consecutive rows are contiguous; used by so_matvec when
  *        one lane owns one row.
  * BINS : rows grouped by nnz into length classes for so_matvec on skewed
- *        matrices, so padding is never streamed. */
-enum { SO_LAYOUT_ROW = 1, SO_LAYOUT_SLOT = 2, SO_LAYOUT_BINS = 4 };
+ *        matrices, so padding is never streamed.
+ * TILED: the nonzeros regrouped by tiles of 256 columns and quads of four rows
+ *        (same values, same ascending order inside every row) for the variant
+ *        of so_matmul that stages X through LDS; costs about 1.3x the ROW
+ *        arrays in HBM.  so_matmul uses it whenever it is present and C is a
+ *        multiple of 4; results are bit-identical to the ROW kernel. */
+enum { SO_LAYOUT_ROW = 1, SO_LAYOUT_SLOT = 2, SO_LAYOUT_BINS = 4, SO_LAYOUT_TILED = 8 };
 
 typedef struct so_ctx so_ctx;         /* one device + one stream + staging arena */
 typedef struct so_ellpack so_ellpack; /* device-resident ELLPACK matrix */

@@ -170,6 +170,208 @@ void launch_act(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, c
     }
 }
 
+// ---------------------------------------------------------------------------
+// LDS-staged variant (SO_LAYOUT_TILED).
+//
+// The row kernel above moves every X operand through the vector L1, which
+// sustains about 50 bytes/clk per CU; LDS sustains three times that for 16-byte
+// reads.  Here a workgroup of 16 waves owns 64 rows and one slab of 64 dense
+// columns, and streams the slab X[:, c0..c0+64) through LDS in tiles of 256 rows
+// (64 KB, double-buffered: the next tile is fetched into registers while the
+// current one is consumed).  A wave works on a quad of four rows, 16 lanes per
+// row, four columns per lane, so one ds_read_b128 per lane serves four FMAs.  The
+// (weight, LDS offset) pairs of a quad's rows for the current tile sit in lanes
+// (chunk of 16 steps per row, fetched one tile ahead and before the X prefetch,
+// so waiting for them never waits for X) and are broadcast inside each 16-lane
+// row with DPP row_newbcast.  Each row still receives its nonzeros in ascending
+// slot order starting from the bias: results are bit-identical to the row kernel.
+// A step that a row of the quad does not have is the pair (0, zero row):
+// fma(0, 0, acc) leaves acc unchanged.
+// ---------------------------------------------------------------------------
+
+constexpr int kTiledWaves = 16;
+constexpr int kMaxChunks = 3;   // chunks of 16 steps held in registers per tile; more run from memory
+
+template <int N>
+__device__ __forceinline__ float bcast_f(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x150 + N, 0xf, 0xf, true));
+}
+template <int N>
+__device__ __forceinline__ uint32_t bcast_u(uint32_t v)
+{
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x150 + N, 0xf, 0xf, true);
+}
+
+// Steps N..END-1 of a chunk: all LDS reads first, then the FMAs in step order.
+template <int N, int END>
+struct StepRange {
+    static __device__ __forceinline__ void read(const char *base, uint32_t eoff, float4 *x)
+    {
+        x[0] = *reinterpret_cast<const float4 *>(base + bcast_u<N>(eoff));
+        StepRange<N + 1, END>::read(base, eoff, x + 1);
+    }
+    static __device__ __forceinline__ void fma(float ew, const float4 *x, float (&acc)[4])
+    {
+        const float w = bcast_f<N>(ew);
+        acc[0] = __builtin_fmaf(w, x[0].x, acc[0]);
+        acc[1] = __builtin_fmaf(w, x[0].y, acc[1]);
+        acc[2] = __builtin_fmaf(w, x[0].z, acc[2]);
+        acc[3] = __builtin_fmaf(w, x[0].w, acc[3]);
+        StepRange<N + 1, END>::fma(ew, x + 1, acc);
+    }
+};
+template <int END>
+struct StepRange<END, END> {
+    static __device__ __forceinline__ void read(const char *, uint32_t, float4 *) {}
+    static __device__ __forceinline__ void fma(float, const float4 *, float (&)[4]) {}
+};
+
+template <int N0, int CNT>
+__device__ __forceinline__ void tiled_steps(const char *base, float ew, uint32_t eoff, float (&acc)[4])
+{
+    float4 x[CNT];
+    StepRange<N0, N0 + CNT>::read(base, eoff, x);
+    StepRange<N0, N0 + CNT>::fma(ew, x, acc);
+}
+
+// One chunk; `left` = steps still to do in this tile (a positive multiple of 4).
+__device__ __forceinline__ void tiled_chunk(const char *base, float ew, uint32_t eoff, uint32_t left, float (&acc)[4])
+{
+    if (left >= 8) {
+        tiled_steps<0, 8>(base, ew, eoff, acc);
+        if (left >= 16) tiled_steps<8, 8>(base, ew, eoff, acc);
+        else if (left >= 12) tiled_steps<8, 4>(base, ew, eoff, acc);
+    } else {
+        tiled_steps<0, 4>(base, ew, eoff, acc);
+    }
+}
+
+template <int ACT>
+__global__ __launch_bounds__(kTiledWaves * 64)
+void ellpack_matmul_tiled_kernel(const so_tile_entry *__restrict__ entries, const so_tile_info *__restrict__ info,
+                                 const uint32_t *__restrict__ quad_rows, uint32_t nquads, uint32_t ntiles,
+                                 uint32_t n, const float *__restrict__ X, uint32_t C,
+                                 const float *__restrict__ bias, float *__restrict__ Y,
+                                 uint32_t nslabs, uint32_t ngroups)
+{
+    constexpr uint32_t KT = so_tiled::kTileRows, ROWB = so_tiled::kSlabCols * 4, TILE = so_tiled::kTileBytes;
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    // Workgroup id -> (column slab, group of 16 quads); an XCD (id % 8) keeps to one
+    // slab when the slab count divides 8, so its L2 holds a single slab of X.
+    uint32_t slab, grp;
+    {
+        const uint32_t xcd = blockIdx.x & 7u, q = blockIdx.x >> 3;
+        if (8 % nslabs == 0) { slab = xcd % nslabs; grp = xcd / nslabs + (8 / nslabs) * q; }
+        else { slab = blockIdx.x % nslabs; grp = blockIdx.x / nslabs; }
+        if (grp >= ngroups) return;
+    }
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t g = lane >> 4, cq = lane & 15u;
+    const uint32_t quad = grp * kTiledWaves + wave;
+    const bool quad_ok = quad < nquads;
+    const uint32_t row = quad_ok ? quad_rows[(size_t)quad * 4 + g] : 0xffffffffu;
+    const uint32_t c0 = slab * so_tiled::kSlabCols;
+    const uint32_t col = c0 + cq * 4;
+
+    float acc[4];
+    {
+        const float b = (bias && row != 0xffffffffu) ? bias[row] : 0.0f;
+        acc[0] = acc[1] = acc[2] = acc[3] = b;
+    }
+
+    // Tile loader: thread -> X row (tid >> 4) + 64*i of the tile, column quad tid & 15.
+    const uint32_t lr = tid >> 4, lc = tid & 15u;
+    const bool lcol_ok = c0 + lc * 4 < C;            // C is a multiple of 4
+    const float *xsrc = X + (size_t)lr * C + c0 + lc * 4;
+    float4 pre[4];
+    auto gload = [&](uint32_t t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t xr = t * KT + lr + 64 * i;
+            pre[i] = (lcol_ok && xr < n) ? *reinterpret_cast<const float4 *>(xsrc + (size_t)(t * KT + 64 * i) * C)
+                                         : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+    };
+    auto lstore = [&](uint32_t buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            *reinterpret_cast<float4 *>(lds + buf * TILE + (lr + 64 * i) * ROWB + lc * 16) = pre[i];
+    };
+
+    const so_tile_info *qi = info + (size_t)(quad_ok ? quad : 0) * ntiles;
+    const so_tile_entry *lane_ent = entries + lane;
+    float ew[kMaxChunks], nw[kMaxChunks];
+    uint32_t eo[kMaxChunks], no[kMaxChunks];
+    auto eload = [&](so_tile_info ti, float (&w)[kMaxChunks], uint32_t (&o)[kMaxChunks]) {
+#pragma unroll
+        for (int c = 0; c < kMaxChunks; ++c) {   // unconditional: the array ends with kMaxChunks spare chunks
+            const so_tile_entry e = lane_ent[(size_t)(ti.chunk0 + c) * 64];
+            w[c] = e.w;
+            o[c] = e.off;
+        }
+    };
+
+    so_tile_info cur = qi[0];
+    if (!quad_ok) cur.steps = 0;
+    eload(cur, ew, eo);
+    if (tid < 16) *reinterpret_cast<float4 *>(lds + so_tiled::kZeroRowOff + tid * 16) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    gload(0);
+    lstore(0);
+    __syncthreads();
+
+    const uint32_t lane_off = cq * 16;
+    for (uint32_t t = 0; t < ntiles; ++t) {
+        so_tile_info nxt{0, 0};
+        if (t + 1 < ntiles) {
+            nxt = qi[t + 1];
+            if (!quad_ok) nxt.steps = 0;
+            eload(nxt, nw, no);
+            gload(t + 1);
+        }
+        const char *base = lds + (t & 1u) * TILE + lane_off;
+#pragma unroll
+        for (int c = 0; c < kMaxChunks; ++c)
+            if (cur.steps > 16u * c) tiled_chunk(base, ew[c], eo[c], cur.steps - 16u * c, acc);
+        for (uint32_t c = kMaxChunks; c * 16u < cur.steps; ++c) {
+            const so_tile_entry e = lane_ent[(size_t)(cur.chunk0 + c) * 64];
+            tiled_chunk(base, e.w, e.off, cur.steps - 16u * c, acc);
+        }
+        if (t + 1 < ntiles) lstore((t + 1) & 1u);
+        __syncthreads();
+        cur = nxt;
+#pragma unroll
+        for (int c = 0; c < kMaxChunks; ++c) { ew[c] = nw[c]; eo[c] = no[c]; }
+    }
+    if (row != 0xffffffffu && col < C) {
+        float4 out;
+        out.x = so_epilogue<ACT>(acc[0]);
+        out.y = so_epilogue<ACT>(acc[1]);
+        out.z = so_epilogue<ACT>(acc[2]);
+        out.w = so_epilogue<ACT>(acc[3]);
+        *reinterpret_cast<float4 *>(Y + (size_t)row * C + col) = out;
+    }
+}
+
+template <int ACT>
+so_status launch_tiled(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, const float *dBias, float *dY)
+{
+    const so_tiled &T = E->tiled;
+    static thread_local bool configured = false;
+    if (!configured) {
+        SO_HIP(hipFuncSetAttribute((const void *)ellpack_matmul_tiled_kernel<ACT>,
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)so_tiled::kLdsBytes));
+        configured = true;
+    }
+    const uint32_t nslabs = so_ceil_div(C, so_tiled::kSlabCols);
+    const uint32_t ngroups = so_ceil_div(T.nquads, kTiledWaves);
+    const uint32_t blocks = (8 % nslabs == 0) ? so_ceil_div(ngroups, 8 / nslabs) * 8 : nslabs * ngroups;
+    ellpack_matmul_tiled_kernel<ACT><<<blocks, kTiledWaves * 64, so_tiled::kLdsBytes, ctx->stream>>>(
+        T.d_entries, T.d_info, T.d_rows, T.nquads, T.ntiles, E->n, dX, C, dBias, dY, nslabs, ngroups);
+    return SO_OK;
+}
+
 } // namespace
 
 extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
@@ -181,8 +383,24 @@ extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX
     SO_REQUIRE(dY != nullptr, "so_matmul: Y is null");
     SO_REQUIRE(dX != nullptr || E->total_nnz == 0, "so_matmul: X is null");
 
-    // Columns per lane: as wide as alignment allows while every tile stays whole.
     const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY;
+    // The LDS-staged kernel needs whole float4 column groups and pays once a slab
+    // of 64 columns is at least a quarter full.
+    if ((E->layouts & SO_LAYOUT_TILED) && C % 4 == 0 && C >= 16 && (align & 15) == 0 &&
+        (size_t)ctx->max_lds_bytes >= so_tiled::kLdsBytes && !getenv("SPARSEOPS_MATMUL_NO_TILED")) {
+        so_status st;
+        switch (act) {
+        case SO_ACT_RELU:    st = launch_tiled<SO_ACT_RELU>(ctx, E, dX, C, dBias, dY); break;
+        case SO_ACT_SIGMOID: st = launch_tiled<SO_ACT_SIGMOID>(ctx, E, dX, C, dBias, dY); break;
+        case SO_ACT_TANH:    st = launch_tiled<SO_ACT_TANH>(ctx, E, dX, C, dBias, dY); break;
+        default:             st = launch_tiled<SO_ACT_NONE>(ctx, E, dX, C, dBias, dY); break;
+        }
+        if (st != SO_OK) return st;
+        SO_LAUNCH_CHECK();
+        return SO_OK;
+    }
+
+    // Columns per lane: as wide as alignment allows while every tile stays whole.
     int vec = 1;
     if (C % 256 == 0 && (align & 15) == 0) vec = 4;
     else if (C % 128 == 0 && (align & 7) == 0) vec = 2;

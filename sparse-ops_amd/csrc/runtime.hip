@@ -246,6 +246,9 @@ static void free_ellpack_arrays(so_ellpack *E)
     if (E->d_idxT) (void)hipFree(E->d_idxT);
     for (auto &b : E->bins)
         if (b.d_rows) (void)hipFree(b.d_rows);
+    if (E->tiled.d_entries) (void)hipFree(E->tiled.d_entries);
+    if (E->tiled.d_info) (void)hipFree(E->tiled.d_info);
+    if (E->tiled.d_rows) (void)hipFree(E->tiled.d_rows);
 }
 
 // Device copy of a host array with 16 zeroed bytes after the last element, so a
@@ -261,6 +264,74 @@ static so_status upload_array(so_ctx *ctx, const T *host, size_t count, T **dev)
     return so_h2d(ctx, p, host, count * sizeof(T));
 }
 
+// K-tiled layout for the LDS-staged matmul (see so_tiled).  Rows are first ordered
+// by stored-nonzero count (longest first, stable) so that the four rows sharing a
+// wavefront have similar lengths; the order only decides which rows share a wave,
+// every row is still written to its own place in Y.
+static so_status build_tiled(so_ctx *ctx, so_ellpack *E, const float *Wd, const uint32_t *idx, const uint32_t *nnz)
+{
+    const uint32_t m = E->m, n = E->n, r = E->r;
+    constexpr uint32_t KT = so_tiled::kTileRows, ROWB = so_tiled::kSlabCols * 4;
+    so_tiled &T = E->tiled;
+    T.nquads = (m + 3) / 4;
+    T.ntiles = std::max(1u, (n + KT - 1) / KT);
+    std::vector<uint32_t> order(m);
+    for (uint32_t i = 0; i < m; ++i) order[i] = i;
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) { return nnz[a] > nnz[b]; });
+    std::vector<uint32_t> qrows((size_t)T.nquads * 4, 0xffffffffu);
+    for (uint32_t i = 0; i < m; ++i) qrows[i] = order[i];
+
+    std::vector<so_tile_info> info((size_t)T.nquads * T.ntiles);
+    std::vector<so_tile_entry> entries;
+    entries.reserve((size_t)E->total_nnz + (size_t)E->total_nnz / 3 + 256);
+    uint64_t total_steps = 0;
+    for (uint32_t q = 0; q < T.nquads; ++q) {
+        uint32_t pos[4] = {0, 0, 0, 0};
+        for (uint32_t t = 0; t < T.ntiles; ++t) {
+            const uint64_t col_end = (uint64_t)(t + 1) * KT;
+            uint32_t cnt[4] = {0, 0, 0, 0}, steps = 0;
+            for (int g = 0; g < 4; ++g) {
+                const uint32_t row = qrows[(size_t)q * 4 + g];
+                if (row == 0xffffffffu) continue;
+                const uint32_t *c = idx + (size_t)row * r;
+                uint32_t p = pos[g];
+                while (p < nnz[row] && c[p] < col_end) ++p;
+                cnt[g] = p - pos[g];
+                steps = std::max(steps, cnt[g]);
+            }
+            steps = (steps + 3u) & ~3u;
+            if (entries.size() / 64 > 0xfffffff0ull) { so_set_error("so_ellpack_upload: matrix too large for the tiled layout"); return SO_ERR_INVALID; }
+            info[(size_t)q * T.ntiles + t] = so_tile_info{(uint32_t)(entries.size() / 64), steps};
+            total_steps += steps;
+            // The zero row sits after both tile buffers; offsets are relative to the buffer the tile uses.
+            const uint32_t zero_off = so_tiled::kZeroRowOff - (t & 1u) * so_tiled::kTileBytes;
+            const uint32_t nch = (steps + 15) / 16;
+            for (uint32_t ch = 0; ch < nch; ++ch)
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t row = qrows[(size_t)q * 4 + g];
+                    for (uint32_t k = 0; k < 16; ++k) {
+                        const uint32_t sidx = ch * 16 + k;
+                        so_tile_entry e{0.0f, zero_off};
+                        if (sidx < cnt[g]) {
+                            const size_t slot = (size_t)row * r + pos[g] + sidx;
+                            e.w = Wd[slot];
+                            e.off = (idx[slot] - t * KT) * ROWB;
+                        }
+                        entries.push_back(e);
+                    }
+                }
+            for (int g = 0; g < 4; ++g) pos[g] += cnt[g];
+        }
+    }
+    // Three zero chunks of slack: the kernel always fetches three chunks per tile.
+    entries.resize(entries.size() + 3 * 64, so_tile_entry{0.0f, so_tiled::kZeroRowOff});
+    T.total_steps = total_steps;
+    so_status s = upload_array(ctx, entries.data(), entries.size(), &T.d_entries);
+    if (s == SO_OK) s = upload_array(ctx, info.data(), info.size(), &T.d_info);
+    if (s == SO_OK) s = upload_array(ctx, qrows.data(), qrows.size(), &T.d_rows);
+    return s;
+}
+
 extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint32_t *idx,
                                        const uint32_t *nnz, uint32_t m, uint32_t n, uint32_t r,
                                        int layouts, so_ellpack **out)
@@ -270,7 +341,7 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
     const size_t slots = (size_t)m * r;
     SO_REQUIRE(m == 0 || nnz != nullptr, "so_ellpack_upload: nnz is null");
     SO_REQUIRE(slots == 0 || (Wd && idx), "so_ellpack_upload: Wd/idx is null");
-    SO_REQUIRE((layouts & ~(SO_LAYOUT_ROW | SO_LAYOUT_SLOT | SO_LAYOUT_BINS)) == 0,
+    SO_REQUIRE((layouts & ~(SO_LAYOUT_ROW | SO_LAYOUT_SLOT | SO_LAYOUT_BINS | SO_LAYOUT_TILED)) == 0,
                "so_ellpack_upload: unknown layout bits 0x%x", layouts);
 
     // Validate on the host before anything reaches a kernel: every stored slot must
@@ -336,6 +407,8 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
             if (!rows[b].empty()) s = upload_array(ctx, rows[b].data(), rows[b].size(), &E->bins[b].d_rows);
         }
     }
+
+    if (s == SO_OK && (layouts & SO_LAYOUT_TILED) && m > 0) s = build_tiled(ctx, E, Wd, idx, nnz);
 
     if (s != SO_OK) {
         free_ellpack_arrays(E);

@@ -25,6 +25,29 @@ struct so_bin {
     uint32_t *d_rows = nullptr;
 };
 
+// K-tiled copy of the matrix for the LDS-staged matmul.  Rows are grouped in
+// quads (four rows share a wavefront, 16 lanes each); the dense operand is consumed
+// in tiles of kTileRows rows.  For every (quad, tile) the nonzeros whose column
+// falls in the tile are stored as "steps": step s holds one (weight, LDS byte
+// offset of the X row inside the tile) pair per row of the quad, padded with
+// (0, offset of a zero row) for rows that have fewer nonzeros in this tile.
+// Steps are stored in chunks of 16: chunk[g][k] is the pair of row g for step k,
+// so the 64 lanes of a wave fetch one chunk with a single coalesced 8-byte load.
+struct so_tile_entry { float w; uint32_t off; };
+struct so_tile_info { uint32_t chunk0; uint32_t steps; };   // steps is a multiple of 4
+struct so_tiled {
+    static constexpr uint32_t kTileRows = 256;   // X rows per LDS tile
+    static constexpr uint32_t kSlabCols = 64;    // dense columns per workgroup
+    static constexpr uint32_t kTileBytes = kTileRows * kSlabCols * 4;
+    static constexpr uint32_t kZeroRowOff = 2 * kTileBytes;      // after the two tile buffers
+    static constexpr uint32_t kLdsBytes = 2 * kTileBytes + kSlabCols * 4;
+    uint32_t nquads = 0, ntiles = 0;
+    uint64_t total_steps = 0;
+    so_tile_entry *d_entries = nullptr;   // [chunks + 3][64]
+    so_tile_info *d_info = nullptr;       // [nquads][ntiles]
+    uint32_t *d_rows = nullptr;           // [nquads*4] row id of each quad member (0xffffffff = none)
+};
+
 struct so_ellpack {
     uint32_t m = 0, n = 0, r = 0;
     uint64_t total_nnz = 0;
@@ -36,6 +59,7 @@ struct so_ellpack {
     float *d_WdT = nullptr;      // [r*m] slot-major (SO_LAYOUT_SLOT)
     uint32_t *d_idxT = nullptr;
     so_bin bins[3];              // SO_LAYOUT_BINS
+    so_tiled tiled;              // SO_LAYOUT_TILED
 };
 
 struct so_graph {

@@ -58,4 +58,8 @@ struct EllpackMirror {
 /// return the device handle.
 const so_ellpack *mirror(const Ellpack &E, int layouts);
 
+/// Device layouts to keep for Y = E * X with C dense columns (ROW, plus TILED
+/// where the LDS-staged kernel pays).
+int matmul_layouts(const Ellpack &E, uint32_t C);
+
 } // namespace sparseops

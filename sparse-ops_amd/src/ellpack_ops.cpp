@@ -17,13 +17,30 @@ Staging &staging()
     return *s;
 }
 
+} // namespace
+
+namespace sparseops {
+// Device layouts worth keeping for Y = E * X with C dense columns: the K-tiled
+// copy (LDS-staged kernel) pays for large, reasonably filled matrices and wide X.
+int matmul_layouts(const Ellpack &E, uint32_t C)
+{
+    uint64_t total = 0;
+    for (uint32_t c : E.nnz) total += c;
+    const bool big = E.m >= 512 && E.n >= 512 && total >= 32ull * E.m;
+    return (big && C >= 32 && C % 4 == 0) ? (SO_LAYOUT_ROW | SO_LAYOUT_TILED) : SO_LAYOUT_ROW;
+}
+} // namespace sparseops
+
+namespace {
+using sparseops::matmul_layouts;
+
 void matmul_host(const Ellpack &E, const float *X, uint32_t C, const float *bias, float *Y, int act)
 {
     using namespace sparseops;
     so_ctx *ctx = context();
     std::lock_guard<std::mutex> lock(context_mutex());
     if (E.m == 0 || C == 0) return;
-    const so_ellpack *dE = mirror(E, SO_LAYOUT_ROW);
+    const so_ellpack *dE = mirror(E, matmul_layouts(E, C));
     Staging &st = staging();
     const std::size_t xbytes = std::size_t(E.n) * C * sizeof(float);
     const std::size_t ybytes = std::size_t(E.m) * C * sizeof(float);

@@ -432,7 +432,7 @@ SparseOnnxModel::SparseOnnxModel(const std::string &onnx_path) : impl_(new Impl(
     std::size_t bias_total = 0;
     for (auto &p : pend) {
         if (p.plan.op != Op::MatMul && p.plan.op != Op::Conv) continue;
-        p.plan.dE = mirror(*p.plan.E, SO_LAYOUT_ROW);
+        p.plan.dE = mirror(*p.plan.E, p.plan.op == Op::MatMul ? matmul_layouts(*p.plan.E, uint32_t(B0)) : SO_LAYOUT_ROW);
         if (p.plan.op == Op::Conv)
             check(so_conv_plan_create(ctx, p.plan.dE, &p.plan.cg, &p.plan.conv), "so_conv_plan_create");
         if (p.plan.has_bias) {

@@ -15,8 +15,8 @@ pytestmark = pytest.mark.gpu
 ACT_TOL = 1e-6
 
 
-def gpu_matmul(ctx, E, X, bias, act="none"):
-    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+def gpu_matmul(ctx, E, X, bias, act="none", layouts=hipabi.LAYOUT_ROW):
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, layouts)
     dX, dY = ctx.array(X), ctx.empty((E.m, X.shape[1]))
     dB = ctx.array(bias) if bias is not None else None
     ctx.matmul(dE, dX, X.shape[1], dB, dY, act)
@@ -90,6 +90,51 @@ def test_matmul_config1_and_config3(ctx, oracle):
     # ... and a permutation of X's columns permutes Y's columns
     perm = np.random.default_rng(0).permutation(256)
     assert np.array_equal(gpu_matmul(ctx, E, np.ascontiguousarray(X[:, perm]), b), Y[:, perm])
+
+
+TILED = hipabi.LAYOUT_ROW | hipabi.LAYOUT_TILED
+
+
+@pytest.mark.parametrize("m,n,C,sp", [(16, 32, 16, .3), (64, 128, 64, .5), (130, 300, 68, .7), (256, 512, 256, .9),
+                                      (1, 1000, 32, .1), (1000, 1, 20, .1), (7, 9, 132, .3), (500, 700, 512, .95),
+                                      (65, 257, 64, 0.), (300, 1000, 20, .5), (67, 1025, 200, .2), (1030, 520, 96, .98)])
+@pytest.mark.parametrize("act", ["none", "relu", "tanh"])
+def test_matmul_lds_tiled_layout(ctx, oracle, m, n, C, sp, act):
+    """The K-tiled device layout (X staged through LDS, four rows per wave) gives the
+    same bits as the row kernel: partial tiles in every dimension, empty rows, a
+    dense row (more steps in a tile than the kernel keeps in registers)."""
+    rng = np.random.default_rng(m * 31 + n * 7 + C)
+    W = sparse_matrix(rng, m, n, sp)
+    if m > 5:
+        W[3] = 0
+        W[m - 2] = rng.standard_normal(n)
+    X = rng.standard_normal((n, C)).astype(np.float32)
+    b = rng.standard_normal(m).astype(np.float32)
+    E = datagen.encode_dense(W)
+    for bias in (b, None):
+        Y, Yo = gpu_matmul(ctx, E, X, bias, act, TILED), oracle.matmul(as_oracle(E), X, bias, act)
+        if act == "tanh":
+            assert rel_err(Y, Yo) <= ACT_TOL
+        else:
+            assert np.array_equal(Y, Yo)
+
+
+def test_matmul_lds_tiled_reference_vectors_and_config3(ctx, oracle, golden):
+    E = datagen.encode_dense(golden["enc_W"])
+    b = golden["mm_bias"]
+    for C in (16, 64, 100, 128, 256):
+        X = golden["mm_X_%d" % C]
+        assert np.array_equal(gpu_matmul(ctx, E, X, b, "none", TILED), golden["mm_Y_%d" % C])
+        assert np.array_equal(gpu_matmul(ctx, E, X, b, "relu", TILED), golden["mm_Yrelu_%d" % C])
+    E, X, b = datagen.config3()
+    Y = gpu_matmul(ctx, E, X, b, "none", TILED)
+    assert np.array_equal(Y, oracle.matmul(as_oracle(E), X, b))
+    assert np.array_equal(Y, gpu_matmul(ctx, E, X, b))                  # row kernel, same bits
+    Xi = X.copy()
+    Xi[0, :] = np.inf                                                   # padded steps must not touch X
+    rows_without_col0 = E.idx[:, 0] != 0
+    Yi = gpu_matmul(ctx, E, Xi, b, "none", TILED)
+    assert np.isfinite(Yi[rows_without_col0]).all() and np.array_equal(Yi[rows_without_col0], Y[rows_without_col0])
 
 
 def test_matmul_degenerate_shapes(ctx, oracle):
