@@ -18,7 +18,6 @@
 namespace {
 
 constexpr int kWavesPerGroup = 4;
-constexpr int kUnroll = 8;
 
 template <int VEC> struct VecT;
 template <> struct VecT<1> { using type = float; };
@@ -72,7 +71,10 @@ __device__ __forceinline__ bool map_tile(const TileMap tm, uint32_t wg, uint32_t
 }
 
 // FULL: every column tile is complete (C % (64*VEC) == 0), no lane predicate.
-template <int VEC, int ACT, bool FULL>
+// kUnroll: gathers per register batch (two batches are in flight).  8 when the
+// chip is full of waves; 32 for launches with only a few waves, where a wave's own
+// memory latency is all there is to hide.
+template <int VEC, int ACT, bool FULL, int kUnroll>
 __global__ __launch_bounds__(kWavesPerGroup * 64)
 void ellpack_matmul_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
                            const uint32_t *__restrict__ nnz, uint32_t m, uint32_t r,
@@ -142,7 +144,7 @@ void ellpack_matmul_kernel(const float *__restrict__ Wd, const uint32_t *__restr
     }
 }
 
-template <int VEC, int ACT>
+template <int VEC, int ACT, int UNROLL = 8>
 void launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, const float *dBias, float *dY)
 {
     TileMap tm;
@@ -153,20 +155,20 @@ void launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, const
     if (tm.mode == 1) blocks = so_ceil_div(tm.nrowgroups, 8u / tm.ntiles) * 8u;
     else blocks = tm.ntiles * tm.nrowgroups;
     const bool full = C % (64u * VEC) == 0;
-    auto k = full ? ellpack_matmul_kernel<VEC, ACT, true> : ellpack_matmul_kernel<VEC, ACT, false>;
+    auto k = full ? ellpack_matmul_kernel<VEC, ACT, true, UNROLL> : ellpack_matmul_kernel<VEC, ACT, false, UNROLL>;
     k<<<blocks, kWavesPerGroup * 64, 0, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->r,
                                                        dX, C, dBias, dY, tm);
 }
 
-template <int VEC>
+template <int VEC, int UNROLL = 8>
 void launch_act(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, const float *dBias,
                 float *dY, int act)
 {
     switch (act) {
-    case SO_ACT_RELU:    launch<VEC, SO_ACT_RELU>(ctx, E, dX, C, dBias, dY); break;
-    case SO_ACT_SIGMOID: launch<VEC, SO_ACT_SIGMOID>(ctx, E, dX, C, dBias, dY); break;
-    case SO_ACT_TANH:    launch<VEC, SO_ACT_TANH>(ctx, E, dX, C, dBias, dY); break;
-    default:             launch<VEC, SO_ACT_NONE>(ctx, E, dX, C, dBias, dY); break;
+    case SO_ACT_RELU:    launch<VEC, SO_ACT_RELU, UNROLL>(ctx, E, dX, C, dBias, dY); break;
+    case SO_ACT_SIGMOID: launch<VEC, SO_ACT_SIGMOID, UNROLL>(ctx, E, dX, C, dBias, dY); break;
+    case SO_ACT_TANH:    launch<VEC, SO_ACT_TANH, UNROLL>(ctx, E, dX, C, dBias, dY); break;
+    default:             launch<VEC, SO_ACT_NONE, UNROLL>(ctx, E, dX, C, dBias, dY); break;
     }
 }
 
@@ -408,7 +410,12 @@ extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX
         const int v = atoi(e);
         if ((v == 1 || v == 2) && v < vec) vec = v;
     }
-    if (vec == 4) launch_act<4>(ctx, E, dX, C, dBias, dY, act);
+    // Few waves in total (at most one per SIMD even with one column per lane): the
+    // launch is latency-bound, so spread it over as many waves as possible and give
+    // each wave 2 x 32 gathers in flight.
+    if ((uint64_t)E->m * so_ceil_div(C, 64) <= 4ull * (uint64_t)ctx->compute_units && E->max_nnz >= 64)
+        launch_act<1, 32>(ctx, E, dX, C, dBias, dY, act);
+    else if (vec == 4) launch_act<4>(ctx, E, dX, C, dBias, dY, act);
     else if (vec == 2) launch_act<2>(ctx, E, dX, C, dBias, dY, act);
     else launch_act<1>(ctx, E, dX, C, dBias, dY, act);
     SO_LAUNCH_CHECK();
