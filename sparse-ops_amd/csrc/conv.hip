@@ -8,9 +8,9 @@
 // materialised: each lane derives (ho, wo, b) from its column once, the plan holds
 // one (offset, dh, dw) triple per stored nonzero, and a tap that falls outside the
 // image leaves the accumulator untouched (src/layers/conv.cpp:62-70).  Waves
-// whose 64 columns are all interior (the common case) skip the bounds tests.
+// whose columns are all interior (the common case) skip the bounds tests.
 //
-// A workgroup is 8 waves = 8 consecutive output channels on the same 64 columns,
+// A workgroup is 8 waves = 8 consecutive output channels on the same columns,
 // so the waves of a workgroup gather from the same input window and share it in
 // the CU's L1.  Accumulation is bias first, then one fused multiply-add per stored
 // nonzero in ascending slot order, as in the reference.
@@ -28,7 +28,27 @@ namespace {
 
 constexpr int kChannelsPerGroup = 8;
 
-template <int ACT>
+template <int VEC> struct ConvVec;
+template <> struct ConvVec<1> { using type = float; };
+template <> struct ConvVec<2> { using type = float2; };
+template <> struct ConvVec<4> { using type = float4; };
+
+template <int VEC>
+__device__ __forceinline__ void conv_load(const float *p, float (&v)[VEC])
+{
+    using T = typename ConvVec<VEC>::type;
+    const T t = *reinterpret_cast<const T *>(p);
+    if constexpr (VEC == 1) { v[0] = t; }
+    if constexpr (VEC == 2) { v[0] = t.x; v[1] = t.y; }
+    if constexpr (VEC == 4) { v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+}
+
+// VEC consecutive columns per lane; B % VEC == 0, so a lane's columns belong to
+// one output pixel (same taps, same bounds test) and are VEC consecutive batch
+// entries: one 4*VEC-byte load per tap.  One batch of 8 taps in flight per wave:
+// a second batch in registers was measured slower (the 8 waves of a workgroup
+// share the input window through L1 and deeper queues evict it).
+template <int VEC, int ACT>
 __global__ __launch_bounds__(kChannelsPerGroup * 64)
 void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict__ taps,
                             const uint32_t *__restrict__ nnz, uint32_t r, so_conv_geom g,
@@ -38,7 +58,7 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t co = __builtin_amdgcn_readfirstlane(blockIdx.y * kChannelsPerGroup + (threadIdx.x >> 6));
     if (co >= g.Cout) return;
-    const uint64_t q = (uint64_t)blockIdx.x * 64u + lane;
+    const uint64_t q = ((uint64_t)blockIdx.x * 64u + lane) * VEC;
     const bool live = q < ncols;
     const uint64_t qq = live ? q : 0;
     const uint32_t p = (uint32_t)(qq / B), b = (uint32_t)(qq % B);
@@ -52,31 +72,76 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
     const uint32_t cnt = nnz[co];
     const float *__restrict__ wrow = Wd + (size_t)co * r;
     const int2 *__restrict__ trow = taps + (size_t)co * r;
-    float acc = bias ? bias[co] : 0.0f;
+    float acc[VEC];
+    {
+        const float b0 = bias ? bias[co] : 0.0f;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = b0;
+    }
 
     if (__all(interior)) {
         const float *__restrict__ xl = X + lanebase;
         uint32_t j = 0;
         for (; j + 8 <= cnt; j += 8) {
-            float w[8], x[8];
+            float w[8], x[8][VEC];
 #pragma unroll
             for (int u = 0; u < 8; ++u) {
                 w[u] = wrow[j + u];
-                x[u] = xl[(int64_t)trow[j + u].x * (int64_t)B];
+                conv_load<VEC>(xl + (int64_t)trow[j + u].x * (int64_t)B, x[u]);
             }
 #pragma unroll
-            for (int u = 0; u < 8; ++u) acc = __builtin_fmaf(w[u], x[u], acc);
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(w[u], x[u][v], acc[v]);
         }
-        for (; j < cnt; ++j) acc = __builtin_fmaf(wrow[j], xl[(int64_t)trow[j].x * (int64_t)B], acc);
+        for (; j < cnt; ++j) {
+            float x[VEC];
+            conv_load<VEC>(xl + (int64_t)trow[j].x * (int64_t)B, x);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(wrow[j], x[v], acc[v]);
+        }
     } else {
         for (uint32_t j = 0; j < cnt; ++j) {
             const int2 t = trow[j];
             const int32_t hin = h0 + (t.y >> 16), win = w0 + (int32_t)(int16_t)(t.y & 0xffff);
-            if ((uint32_t)hin < g.H_in && (uint32_t)win < g.W_in)
-                acc = __builtin_fmaf(wrow[j], X[lanebase + (int64_t)t.x * (int64_t)B], acc);
+            if ((uint32_t)hin < g.H_in && (uint32_t)win < g.W_in) {
+                float x[VEC];
+                conv_load<VEC>(X + lanebase + (int64_t)t.x * (int64_t)B, x);
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(wrow[j], x[v], acc[v]);
+            }
         }
     }
-    if (live) Y[(size_t)co * ncols + q] = so_epilogue<ACT>(acc);
+    if (live) {
+        using T = typename ConvVec<VEC>::type;
+        T out;
+        if constexpr (VEC == 1) { out = so_epilogue<ACT>(acc[0]); }
+        if constexpr (VEC == 2) { out.x = so_epilogue<ACT>(acc[0]); out.y = so_epilogue<ACT>(acc[1]); }
+        if constexpr (VEC == 4) {
+            out.x = so_epilogue<ACT>(acc[0]); out.y = so_epilogue<ACT>(acc[1]);
+            out.z = so_epilogue<ACT>(acc[2]); out.w = so_epilogue<ACT>(acc[3]);
+        }
+        *reinterpret_cast<T *>(Y + (size_t)co * ncols + q) = out;
+    }
+}
+
+template <int VEC>
+void conv_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B, uint64_t ncols,
+                 const float *dBias, float *dY, int act)
+{
+    const so_conv_geom &g = plan->g;
+    const so_ellpack *E = plan->E;
+    const dim3 grid((uint32_t)((ncols + 64ull * VEC - 1) / (64ull * VEC)), so_ceil_div(g.Cout, kChannelsPerGroup));
+#define SO_CONV_LAUNCH(A)                                                                          \
+    conv2d_implicit_kernel<VEC, A><<<grid, kChannelsPerGroup * 64, 0, ctx->stream>>>(              \
+        E->d_Wd, plan->d_taps, E->d_nnz, E->r, g, dX, B, ncols, dBias, dY)
+    switch (act) {
+    case SO_ACT_RELU:    SO_CONV_LAUNCH(SO_ACT_RELU); break;
+    case SO_ACT_SIGMOID: SO_CONV_LAUNCH(SO_ACT_SIGMOID); break;
+    case SO_ACT_TANH:    SO_CONV_LAUNCH(SO_ACT_TANH); break;
+    default:             SO_CONV_LAUNCH(SO_ACT_NONE); break;
+    }
+#undef SO_CONV_LAUNCH
 }
 
 } // namespace
@@ -153,20 +218,12 @@ extern "C" so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const floa
     const uint64_t ncols = (uint64_t)g.H_out * g.W_out * B;
     if (g.Cout == 0 || ncols == 0) return SO_OK;
     SO_REQUIRE(dX && dY, "so_conv2d: null tensor");
-    const uint64_t xtiles = (ncols + 63) / 64;
-    SO_REQUIRE(xtiles < (1ull << 31), "so_conv2d: output plane too large");
-    const dim3 grid((uint32_t)xtiles, so_ceil_div(g.Cout, kChannelsPerGroup));
-    const so_ellpack *E = plan->E;
-#define SO_CONV_LAUNCH(A)                                                                          \
-    conv2d_implicit_kernel<A><<<grid, kChannelsPerGroup * 64, 0, ctx->stream>>>(                   \
-        E->d_Wd, plan->d_taps, E->d_nnz, E->r, g, dX, B, ncols, dBias, dY)
-    switch (act) {
-    case SO_ACT_RELU:    SO_CONV_LAUNCH(SO_ACT_RELU); break;
-    case SO_ACT_SIGMOID: SO_CONV_LAUNCH(SO_ACT_SIGMOID); break;
-    case SO_ACT_TANH:    SO_CONV_LAUNCH(SO_ACT_TANH); break;
-    default:             SO_CONV_LAUNCH(SO_ACT_NONE); break;
-    }
-#undef SO_CONV_LAUNCH
+    SO_REQUIRE((ncols + 63) / 64 < (1ull << 31), "so_conv2d: output plane too large");
+    // Batch entries per lane: as many as divide B and keep 16/8-byte alignment.
+    const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY;
+    if (B % 4 == 0 && (align & 15) == 0) conv_launch<4>(ctx, plan, dX, B, ncols, dBias, dY, act);
+    else if (B % 2 == 0 && (align & 7) == 0) conv_launch<2>(ctx, plan, dX, B, ncols, dBias, dY, act);
+    else conv_launch<1>(ctx, plan, dX, B, ncols, dBias, dY, act);
     SO_LAUNCH_CHECK();
     return SO_OK;
 }

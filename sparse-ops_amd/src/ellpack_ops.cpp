@@ -27,7 +27,7 @@ int matmul_layouts(const Ellpack &E, uint32_t C)
     uint64_t total = 0;
     for (uint32_t c : E.nnz) total += c;
     const bool big = E.m >= 512 && E.n >= 512 && total >= 32ull * E.m;
-    return (big && C >= 32 && C % 4 == 0) ? (SO_LAYOUT_ROW | SO_LAYOUT_TILED) : SO_LAYOUT_ROW;
+    return (big && C >= 64 && C % 4 == 0) ? (SO_LAYOUT_ROW | SO_LAYOUT_TILED) : SO_LAYOUT_ROW;
 }
 } // namespace sparseops
 
