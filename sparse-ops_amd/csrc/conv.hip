@@ -16,6 +16,7 @@
 // nonzero in ascending slot order, as in the reference.
 #include "so_internal.h"
 
+#include <cstdlib>
 #include <new>
 
 struct so_conv_plan {
@@ -101,7 +102,29 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
             for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(wrow[j], x[v], acc[v]);
         }
     } else {
-        for (uint32_t j = 0; j < cnt; ++j) {
+        // Some lane of the wave has taps outside the image.  Same batches of 8, without
+        // branches: a tap that is out of bounds for a lane loads a harmless in-bounds
+        // address (the lane's own batch entry of pixel (0,0,0)) and contributes
+        // fma(w, 0, acc) = acc, which is what skipping it gives.
+        const float *__restrict__ xsafe = X + b;
+        uint32_t j = 0;
+        for (; j + 8 <= cnt; j += 8) {
+            float w[8], x[8][VEC];
+            bool ok[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int2 t = trow[j + u];
+                w[u] = wrow[j + u];
+                const int32_t hin = h0 + (t.y >> 16), win = w0 + (int32_t)(int16_t)(t.y & 0xffff);
+                ok[u] = (uint32_t)hin < g.H_in && (uint32_t)win < g.W_in;
+                conv_load<VEC>(ok[u] ? X + lanebase + (int64_t)t.x * (int64_t)B : xsafe, x[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(w[u], ok[u] ? x[u][v] : 0.0f, acc[v]);
+        }
+        for (; j < cnt; ++j) {
             const int2 t = trow[j];
             const int32_t hin = h0 + (t.y >> 16), win = w0 + (int32_t)(int16_t)(t.y & 0xffff);
             if ((uint32_t)hin < g.H_in && (uint32_t)win < g.W_in) {
@@ -221,8 +244,10 @@ extern "C" so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const floa
     SO_REQUIRE((ncols + 63) / 64 < (1ull << 31), "so_conv2d: output plane too large");
     // Batch entries per lane: as many as divide B and keep 16/8-byte alignment.
     const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY;
-    if (B % 4 == 0 && (align & 15) == 0) conv_launch<4>(ctx, plan, dX, B, ncols, dBias, dY, act);
-    else if (B % 2 == 0 && (align & 7) == 0) conv_launch<2>(ctx, plan, dX, B, ncols, dBias, dY, act);
+    int maxvec = 4;
+    if (const char *e = getenv("SPARSEOPS_CONV_VEC")) maxvec = atoi(e);
+    if (maxvec >= 4 && B % 4 == 0 && (align & 15) == 0) conv_launch<4>(ctx, plan, dX, B, ncols, dBias, dY, act);
+    else if (maxvec >= 2 && B % 2 == 0 && (align & 7) == 0) conv_launch<2>(ctx, plan, dX, B, ncols, dBias, dY, act);
     else conv_launch<1>(ctx, plan, dX, B, ncols, dBias, dY, act);
     SO_LAUNCH_CHECK();
     return SO_OK;
