@@ -386,10 +386,19 @@ extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX
     SO_REQUIRE(dX != nullptr || E->total_nnz == 0, "so_matmul: X is null");
 
     const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY;
-    // The LDS-staged kernel needs whole float4 column groups and pays once a slab
-    // of 64 columns is at least a quarter full.
-    if ((E->layouts & SO_LAYOUT_TILED) && C % 4 == 0 && C >= 16 && (align & 15) == 0 &&
-        (size_t)ctx->max_lds_bytes >= so_tiled::kLdsBytes && !getenv("SPARSEOPS_MATMUL_NO_TILED")) {
+    // The LDS-staged kernel needs whole float4 column groups.  It takes one
+    // workgroup per (64 rows, 64 columns), one workgroup per CU at a time, so it pays
+    // only when that grid covers most of the chip; smaller problems stay on the row
+    // kernel (SPARSEOPS_MATMUL_TILED=1 forces it, =0 forbids it: tuning and tests).
+    bool tiled = (E->layouts & SO_LAYOUT_TILED) && C % 4 == 0 && C >= 16 && (align & 15) == 0 &&
+                 (size_t)ctx->max_lds_bytes >= so_tiled::kLdsBytes;
+    if (tiled) {
+        const uint64_t groups = (uint64_t)so_ceil_div(C, so_tiled::kSlabCols) * so_ceil_div(E->tiled.nquads, kTiledWaves);
+        const char *force = getenv("SPARSEOPS_MATMUL_TILED");
+        if (force) tiled = force[0] == '1';
+        else tiled = 4 * groups >= 3 * (uint64_t)ctx->compute_units;
+    }
+    if (tiled) {
         so_status st;
         switch (act) {
         case SO_ACT_RELU:    st = launch_tiled<SO_ACT_RELU>(ctx, E, dX, C, dBias, dY); break;
