@@ -125,7 +125,48 @@ def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup
     return out
 
 
-def bench_mlp(steps, warmup):
+def cpu_baseline_mlp(Ws, X, y_gpu, runs=10):
+    """The same MLP forward on the host cores with the reference's kernels, as its
+    runtime chains them (src/model_run.cpp:28-127): ellpack_matmul_fused with the
+    fused ReLU, then the separate scalar Sigmoid / Tanh layers
+    (src/layers/activation.cpp:22-62).  Falls back to the plain-C restatement."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    from oracle import Oracle, Ref
+    A0 = np.ascontiguousarray(X.T)
+    acts = ["relu", "sigmoid", "tanh", None]
+    if Ref.available():
+        ref, kind = Ref(), "reference"
+        hs = [ref.encode(W) for W in Ws]
+
+        def forward():
+            A = A0
+            for h, act in zip(hs, acts):
+                A = ref.matmul_fused(h, A, None, use_mask=False, fuse_relu=(act == "relu"))
+                if act in ("sigmoid", "tanh"):
+                    A = ref.act_inplace(A, act)
+            return A
+    else:
+        orc, kind = Oracle(), "port"
+        Es = [orc.encode(W) for W in Ws]
+
+        def forward():
+            A = A0
+            for E, act in zip(Es, acts):
+                A = orc.matmul(E, A, None, act or "none")
+            return A
+    Y = forward()
+    times = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        forward()
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    return {"samples_per_s": round(X.shape[0] / med, 1), "ms_per_batch": round(med * 1e3, 3), "kind": kind,
+            "cores": int(os.environ.get("OMP_NUM_THREADS", len(os.sched_getaffinity(0)))),
+            "gpu_max_rel_err_vs_cpu": float(np.abs(Y.T.astype(np.float64) - y_gpu).max() / max(np.abs(Y).max(), 1e-30))}
+
+
+def bench_mlp(steps, warmup, with_cpu=True):
     import datagen
     import onnx_wire as ow
     import sparseops_backend as sb
@@ -141,7 +182,9 @@ def bench_mlp(steps, warmup):
         model.run(Xf)                       # includes H2D of the input and D2H of the output
     dt = (time.perf_counter() - t0) / steps
     dev_ms = model.time_device(steps, warmup)   # chain only, activations resident in HBM
-    return {"workload": "MLP 784-4096-4096-4096-10, 90% sparse, B=256", "layers": model.describe(),
+    y_gpu = model.run(Xf)
+    cpu = cpu_baseline_mlp(Ws, X, y_gpu) if with_cpu else None
+    return {"workload": "MLP 784-4096-4096-4096-10, 90% sparse, B=256", "layers": model.describe(), "cpu_baseline": cpu,
             "samples_per_s_device_resident": round(256 / (dev_ms * 1e-3), 1), "us_per_batch_device_resident": round(dev_ms * 1e3, 2),
             "samples_per_s_host_to_host": round(256 / dt, 1), "us_per_batch_host_to_host": round(dt * 1e6, 2),
             "nnz_gflops_device_resident": round(model.nnz_flops_per_sample() * 256 / (dev_ms * 1e-3) / 1e9, 1)}
@@ -243,7 +286,7 @@ def main():
                                              datagen.config2b, hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS, hipabi.LAYOUT_BINS,
                                              k, args.warmup)
         log("sparse MLP ...")
-        extras["mlp"] = bench_mlp(k, args.warmup)
+        extras["mlp"] = bench_mlp(k, args.warmup, with_cpu=not args.no_cpu)
         log("sparse CNN ...")
         extras["cnn"] = bench_cnn(max(5, args.steps // 20), 2)
         result["extras"] = extras
