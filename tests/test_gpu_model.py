@@ -252,3 +252,28 @@ def test_resnet18_shaped(backend, oracle, tmp_path):
     assert np.array_equal(Y, Yo)
     Yt = torch_resnet(t, X, width=32)
     assert rel_err(Y, Yt) <= 1e-5 and np.allclose(Y, Yt, atol=1e-4)
+
+
+@pytest.mark.parametrize("name", ["mlp_gemm", "cnn_gap", "cnn_flatten_fc", "resnet_tiny"])
+def test_torch_exported_models(backend, oracle, name):
+    """Real `torch.onnx.export` files (tests/golden/torch_export, the topologies of the
+    reference's tests/full_test.py, tests/test_cnn.py and tests/test_resnet.py) against
+    PyTorch's own output (the reference's atol=1e-4) and the oracle chain."""
+    from graph_oracle import run_graph
+    d = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "torch_export")
+    exp = np.load(os.path.join(d, "expected.npz"))
+    X, Yt = exp[name + "__input"], exp[name + "__output"]
+    path = os.path.join(d, name + ".onnx")
+    model = backend.SparseOnnxModel(path)
+    assert model.output_shape() == list(Yt.shape)
+    Y = model.run(X)
+    assert Y.shape == Yt.shape
+    assert rel_err(Y, Yt) <= 1e-5 and np.allclose(Y, Yt, atol=1e-4)
+    Yo = run_graph(oracle, open(path, "rb").read(), X)
+    if name in ("cnn_gap", "resnet_tiny"):      # only exact layers (conv, ReLU, pools, add, FC)
+        assert np.array_equal(Y, Yo)
+    else:                                       # sigmoid / tanh: device libm vs glibc
+        assert rel_err(Y, Yo) <= 1e-6
+    # a second batch through the same model object, in Fortran order
+    Y2 = model.run(np.asfortranarray(X[::-1].copy()))
+    assert rel_err(Y2, Yt[::-1]) <= 1e-5

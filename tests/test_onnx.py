@@ -3,6 +3,8 @@
 error behaviour.  The writer is cross-checked against an independent encoder:
 google.protobuf dynamic messages built from a descriptor of the same onnx.proto
 fields."""
+import os
+
 import numpy as np
 import pytest
 
@@ -166,3 +168,50 @@ def test_valid_model_without_gpu_fails_loudly(backend, tmp_path):
                                                        [("y", (2, 3))], [("W", W)]))
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         backend.SparseOnnxModel(path)
+
+
+# Real `torch.onnx.export` output (TorchScript exporter, opset 14), written once by
+# tests/golden/make_torch_onnx.py together with PyTorch's own outputs.
+TORCH_EXPORTS = {
+    "mlp_gemm": ["Gemm", "Relu", "Gemm", "Sigmoid", "Gemm", "Tanh", "Gemm"],
+    "cnn_gap": ["Conv", "Relu", "MaxPool", "Conv", "Relu", "GlobalAveragePool", "Flatten", "Gemm"],
+    "cnn_flatten_fc": ["Conv", "Relu", "MaxPool", "Conv", "Tanh", "Flatten", "Gemm", "Relu", "Gemm"],
+    "resnet_tiny": None,
+}
+EXPORT_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "torch_export")
+
+
+@pytest.mark.parametrize("name", sorted(TORCH_EXPORTS))
+def test_torch_exported_graph_parses(backend, name):
+    """Both wire readers on files the builder's writer did not produce."""
+    path = os.path.join(EXPORT_DIR, name + ".onnx")
+    exp = np.load(os.path.join(EXPORT_DIR, "expected.npz"))
+    m = backend.parse_onnx(path)
+    mp = ow.read_model(open(path, "rb").read())
+    ops = [n["op_type"] for n in m["nodes"]]
+    assert ops == [n["op_type"] for n in mp["nodes"]]
+    if TORCH_EXPORTS[name] is not None:
+        assert ops == TORCH_EXPORTS[name]
+    else:   # BatchNorm folded into the convolutions; 2 + 2 basic blocks, one projection
+        assert ops.count("Conv") == 10 and ops.count("Add") == 4 and "BatchNormalization" not in ops
+    assert m["inputs"] == [("input", exp[name + "__input"].shape)]
+    assert m["outputs"] == [("output", exp[name + "__output"].shape)]
+    assert sorted(m["initializers"]) == sorted(mp["initializers"])
+    for k, v in mp["initializers"].items():
+        assert np.array_equal(m["initializers"][k], v), k
+    for a, b in zip(m["nodes"], mp["nodes"]):
+        assert a["input"] == b["input"] and a["output"] == b["output"] and a["attrs"] == b["attrs"]
+
+
+@pytest.mark.parametrize("name", sorted(TORCH_EXPORTS))
+def test_torch_exported_graph_through_the_oracle_chain(oracle, name):
+    """The oracle's layer chain over the exported graph reproduces PyTorch's output,
+    which pins the graph semantics the GPU tests compare against (Gemm transB + bias,
+    Flatten of a 4-D tensor into an FC, folded BatchNorm, residual Add)."""
+    from graph_oracle import run_graph
+    exp = np.load(os.path.join(EXPORT_DIR, "expected.npz"))
+    payload = open(os.path.join(EXPORT_DIR, name + ".onnx"), "rb").read()
+    Y = run_graph(oracle, payload, exp[name + "__input"])
+    Yt = exp[name + "__output"]
+    assert Y.shape == Yt.shape
+    assert np.abs(Y - Yt).max() / np.abs(Yt).max() <= 1e-5 and np.allclose(Y, Yt, atol=1e-4)
