@@ -304,6 +304,7 @@ static so_status build_tiled(so_ctx *ctx, so_ellpack *E, const float *Wd, const 
             info[(size_t)q * T.ntiles + t] = so_tile_info{(uint32_t)(entries.size() / 64), steps};
             total_steps += steps;
             // The zero row sits after both tile buffers; offsets are relative to the buffer the tile uses.
+            // A padding step is fma(-0, +0, acc): adding -0 leaves every accumulator, -0 included, as it is.
             const uint32_t zero_off = so_tiled::kZeroRowOff - (t & 1u) * so_tiled::kTileBytes;
             const uint32_t nch = (steps + 15) / 16;
             for (uint32_t ch = 0; ch < nch; ++ch)
@@ -311,7 +312,7 @@ static so_status build_tiled(so_ctx *ctx, so_ellpack *E, const float *Wd, const 
                     const uint32_t row = qrows[(size_t)q * 4 + g];
                     for (uint32_t k = 0; k < 16; ++k) {
                         const uint32_t sidx = ch * 16 + k;
-                        so_tile_entry e{0.0f, zero_off};
+                        so_tile_entry e{-0.0f, zero_off};
                         if (sidx < cnt[g]) {
                             const size_t slot = (size_t)row * r + pos[g] + sidx;
                             e.w = Wd[slot];
@@ -324,7 +325,7 @@ static so_status build_tiled(so_ctx *ctx, so_ellpack *E, const float *Wd, const 
         }
     }
     // Three zero chunks of slack: the kernel always fetches three chunks per tile.
-    entries.resize(entries.size() + 3 * 64, so_tile_entry{0.0f, so_tiled::kZeroRowOff});
+    entries.resize(entries.size() + 3 * 64, so_tile_entry{-0.0f, so_tiled::kZeroRowOff});
     T.total_steps = total_steps;
     so_status s = upload_array(ctx, entries.data(), entries.size(), &T.d_entries);
     if (s == SO_OK) s = upload_array(ctx, info.data(), info.size(), &T.d_info);

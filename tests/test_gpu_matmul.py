@@ -149,6 +149,25 @@ def test_matmul_lds_tiled_reference_vectors_and_config3(ctx, oracle, golden):
     assert np.isfinite(Yi[rows_without_col0]).all() and np.array_equal(Yi[rows_without_col0], Y[rows_without_col0])
 
 
+def test_matmul_lds_tiled_keeps_negative_zero(ctx, oracle):
+    """Rows that share a wave with longer rows run padding steps; those must leave a
+    -0.0 accumulator (bias -0.0, no contribution yet) as it is, sign bit included."""
+    rng = np.random.default_rng(5)
+    W = sparse_matrix(rng, 64, 512, .8)
+    W[::3] = 0                                   # empty rows next to populated ones
+    W[1, :] = 0
+    W[1, 7] = 2.0                                # one nonzero, late K-tiles are padding only
+    X = rng.standard_normal((512, 64)).astype(np.float32)
+    X[7, :] = -0.0                               # 2 * -0 = -0 on top of bias -0
+    b = np.full(64, -0.0, np.float32)
+    E = datagen.encode_dense(W)
+    Yo = oracle.matmul(as_oracle(E), X, b)
+    assert np.signbit(Yo[0]).all() and np.signbit(Yo[1]).all()
+    for layouts in (TILED, hipabi.LAYOUT_ROW):
+        Y = gpu_matmul(ctx, E, X, b, "none", layouts)
+        assert np.array_equal(Y, Yo) and np.array_equal(np.signbit(Y), np.signbit(Yo))
+
+
 def test_matmul_degenerate_shapes(ctx, oracle):
     # zero-sized launches are early-outs, not HIP errors
     for (m, n, C) in [(0, 0, 0), (0, 5, 3), (5, 0, 3), (5, 4, 0)]:
