@@ -153,6 +153,11 @@ typedef struct so_conv_plan so_conv_plan;
 so_status so_conv_plan_create(so_ctx *ctx, const so_ellpack *E, const so_conv_geom *g,
                               so_conv_plan **out);
 so_status so_conv_plan_free(so_ctx *ctx, so_conv_plan *plan);
+/* The LDS-windowed kernel's parameters for this plan (no counterpart in the reference:
+ * a tuning/inspection aid): out = {tile_h, tile_w, window_h, window_w, channels per
+ * chunk, chunks, output channels per wave, 0}; all zero when the geometry does not
+ * suit that kernel and so_conv2d always takes the gather kernel. */
+so_status so_conv_plan_window(const so_conv_plan *plan, uint32_t out[8]);
 
 /* Sparse convolution by implicit im2col: conv2d_implicit_im2col_fmajor
  * (src/layers/conv.cpp:16-108), on the [C][H][W][B] layout of

@@ -16,13 +16,29 @@
 // nonzero in ascending slot order, as in the reference.
 #include "so_internal.h"
 
+#include <algorithm>
 #include <cstdlib>
+#include <cstring>
 #include <new>
+#include <vector>
+
+// What the LDS-windowed kernel needs on top of the plan; built only for geometries it suits.
+// The input channels are cut into chunks of `cc`; for one chunk and one tile of TH x TW output
+// pixels the input window is IH x IW pixels.  A stored nonzero becomes {weight bits, pixel
+// offset of its tap inside the chunk's window}; cstart[co*(nch+1) + t] is the slot at which
+// chunk t begins in row co (slots are ordered by input channel, so chunks are slot ranges).
+struct so_conv_window {
+    uint32_t TH = 0, TW = 0, IH = 0, IW = 0, cc = 0, nch = 0, tiles_x = 0, tiles_y = 0;
+    int cpw = 0;                  // output channels per wave: 4 or 2 (8 would spill registers)
+    int2 *d_went = nullptr;       // [Cout * r]
+    uint32_t *d_cstart = nullptr; // [Cout * (nch + 1)]
+};
 
 struct so_conv_plan {
     so_conv_geom g;
     const so_ellpack *E = nullptr;
     int2 *d_taps = nullptr;  // per slot: x = (cin*H + dh)*W + dw (elements of B floats), y = dh<<16 | (dw & 0xffff)
+    so_conv_window win;      // win.cc == 0: not built
 };
 
 namespace {
@@ -148,6 +164,248 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
     }
 }
 
+
+// ---- LDS-windowed variant -------------------------------------------------------------
+//
+// A workgroup of 16 waves owns a tile of TH x TW output pixels x BT batch entries and a block
+// of output channels.  It walks the input channels in chunks; a chunk's input window (halo
+// included, out-of-image pixels as zeros) is copied to LDS once and every tap of every output
+// channel of the block is then a 16-byte LDS read, about three times the rate the L1 gathers
+// of the kernel above sustain.  Lanes: LPP = BT/4 lanes per pixel (4 batch entries each), so a
+// wave covers 64/LPP pixels; the 16 waves are PG pixel groups x CG channel groups and a wave
+// accumulates CPW output channels.  The chunk's nonzeros of one output channel (at most 64)
+// sit one per lane in a register pair and are handed to the whole wave with v_readlane, so the
+// weight is a scalar operand and the tap offset a scalar addend.  Per output the multiply-adds
+// run in slot order (chunks ascend, slots ascend inside a chunk): same bits as the kernel above.
+// Windows are double-buffered: chunk t+1 is fetched into registers while chunk t is computed.
+constexpr int kWinThreads = 1024;
+constexpr int kWinMaxPerThread = 6;   // float4 window elements a thread copies per chunk
+
+struct WinArgs {
+    uint32_t TH, TW, IH, IW, cc, nch, tiles_x, pg, cg, win_f4, r;
+};
+
+template <int CPW, int LPP, int ACT>
+__global__ __launch_bounds__(kWinThreads)
+void conv2d_window_kernel(const int2 *__restrict__ went, const uint32_t *__restrict__ cstart, WinArgs a, so_conv_geom g,
+                          const float *__restrict__ X, uint32_t B, const float *__restrict__ bias, float *__restrict__ Y)
+{
+    extern __shared__ float4 win_lds[];
+    constexpr uint32_t BT = LPP * 4, PPW = 64 / LPP, SHIFT = (LPP == 8 ? 7 : LPP == 4 ? 6 : LPP == 2 ? 5 : 4);
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t pgi = wave % a.pg, cgi = wave / a.pg;             // waves with cgi >= cg only help copying
+    const uint32_t th0 = (blockIdx.x / a.tiles_x) * a.TH, tw0 = (blockIdx.x % a.tiles_x) * a.TW;
+    const uint32_t co0 = (blockIdx.y * a.cg + cgi) * CPW;
+    const uint32_t bz = blockIdx.z * BT;
+    const bool computes = cgi < a.cg;
+
+    // this lane's output pixel and its corner inside the window
+    const uint32_t pl = pgi * PPW + lane / LPP, b4 = lane % LPP;
+    const bool pvalid = pl < a.TH * a.TW;
+    const uint32_t pc = pvalid ? pl : 0u;
+    const uint32_t ty = pc / a.TW, tx = pc % a.TW;
+    const bool live = computes && pvalid && th0 + ty < g.H_out && tw0 + tx < g.W_out;
+    const uint32_t lanebase = ((ty * g.stride_h * a.IW + tx * g.stride_w) << SHIFT) + b4 * 16u;   // bytes
+    const uint32_t buf_bytes = a.win_f4 * 16u;
+
+    // window elements this thread copies: element e = tid + k*1024 is float4 (cl, ih, iw, b4)
+    int32_t goff[kWinMaxPerThread];      // float offset from the chunk's first channel; -1: outside the image
+    uint32_t gcl[kWinMaxPerThread];      // channel inside the chunk; 0xffffffff: no such element
+#pragma unroll
+    for (int k = 0; k < kWinMaxPerThread; ++k) {
+        const uint32_t e = tid + (uint32_t)k * kWinThreads;
+        goff[k] = -1;
+        gcl[k] = 0xffffffffu;
+        if (e < a.win_f4) {
+            const uint32_t eb = e % LPP, px = e / LPP;
+            const uint32_t iw = px % a.IW, rest = px / a.IW, ih = rest % a.IH, cl = rest / a.IH;
+            const int32_t gh = (int32_t)(th0 * g.stride_h + ih) - (int32_t)g.pad_h;
+            const int32_t gw = (int32_t)(tw0 * g.stride_w + iw) - (int32_t)g.pad_w;
+            gcl[k] = cl;
+            if ((uint32_t)gh < g.H_in && (uint32_t)gw < g.W_in)
+                goff[k] = (int32_t)(((cl * g.H_in + (uint32_t)gh) * g.W_in + (uint32_t)gw) * B + bz + eb * 4u);
+        }
+    }
+    const size_t chunk_floats = (size_t)a.cc * g.H_in * g.W_in * B;
+
+    float4 xr[kWinMaxPerThread];
+    auto fetch_window = [&](uint32_t t) {
+        const float *__restrict__ Xc = X + (size_t)t * chunk_floats;
+        const uint32_t cleft = g.Cin - t * a.cc;                       // channels left from this chunk on
+#pragma unroll
+        for (int k = 0; k < kWinMaxPerThread; ++k) {
+            xr[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (goff[k] >= 0 && gcl[k] < cleft) xr[k] = *reinterpret_cast<const float4 *>(Xc + goff[k]);
+        }
+    };
+    auto store_window = [&](uint32_t buf) {
+#pragma unroll
+        for (int k = 0; k < kWinMaxPerThread; ++k)
+            if (gcl[k] != 0xffffffffu) win_lds[buf * a.win_f4 + tid + (uint32_t)k * kWinThreads] = xr[k];
+    };
+
+    // the chunk's nonzeros of each of this wave's output channels, one per lane
+    uint32_t ecnt[CPW], ncnt[CPW];
+    int2 ent[CPW], nent[CPW];
+    auto fetch_entries = [&](uint32_t t, uint32_t (&cnt)[CPW], int2 (&e)[CPW]) {
+#pragma unroll
+        for (int c = 0; c < CPW; ++c) {
+            const uint32_t co = co0 + c;
+            cnt[c] = 0;
+            e[c] = make_int2(0, 0);
+            if (computes && co < g.Cout) {
+                const uint32_t s0 = cstart[(size_t)co * (a.nch + 1) + t], s1 = cstart[(size_t)co * (a.nch + 1) + t + 1];
+                cnt[c] = s1 - s0;
+                if (lane < cnt[c]) e[c] = went[(size_t)co * a.r + s0 + lane];
+            }
+        }
+    };
+
+    float acc[CPW][4];
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+        const float b0 = (bias && computes && co0 + c < g.Cout) ? bias[co0 + c] : 0.0f;
+        acc[c][0] = acc[c][1] = acc[c][2] = acc[c][3] = b0;
+    }
+
+    fetch_window(0);
+    fetch_entries(0, ecnt, ent);
+    store_window(0);
+    __syncthreads();
+
+    const char *lds_bytes = reinterpret_cast<const char *>(win_lds);
+    for (uint32_t t = 0; t < a.nch; ++t) {
+        const bool more = t + 1 < a.nch;
+        if (more) {
+            fetch_window(t + 1);
+            fetch_entries(t + 1, ncnt, nent);
+        }
+        const uint32_t base = lanebase + (t & 1u) * buf_bytes;
+#pragma unroll
+        for (int c = 0; c < CPW; ++c) {
+            const uint32_t cnt = ecnt[c];
+            const int wbits = ent[c].x, offs = ent[c].y;
+            uint32_t e = 0;
+            for (; e + 4 <= cnt; e += 4) {
+                float w[4];
+                float4 x[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    w[u] = __int_as_float(__builtin_amdgcn_readlane(wbits, (int)(e + u)));
+                    const uint32_t o = (uint32_t)__builtin_amdgcn_readlane(offs, (int)(e + u));
+                    x[u] = *reinterpret_cast<const float4 *>(lds_bytes + base + (o << SHIFT));
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    acc[c][0] = __builtin_fmaf(w[u], x[u].x, acc[c][0]);
+                    acc[c][1] = __builtin_fmaf(w[u], x[u].y, acc[c][1]);
+                    acc[c][2] = __builtin_fmaf(w[u], x[u].z, acc[c][2]);
+                    acc[c][3] = __builtin_fmaf(w[u], x[u].w, acc[c][3]);
+                }
+            }
+            for (; e < cnt; ++e) {
+                const float w = __int_as_float(__builtin_amdgcn_readlane(wbits, (int)e));
+                const uint32_t o = (uint32_t)__builtin_amdgcn_readlane(offs, (int)e);
+                const float4 x = *reinterpret_cast<const float4 *>(lds_bytes + base + (o << SHIFT));
+                acc[c][0] = __builtin_fmaf(w, x.x, acc[c][0]);
+                acc[c][1] = __builtin_fmaf(w, x.y, acc[c][1]);
+                acc[c][2] = __builtin_fmaf(w, x.z, acc[c][2]);
+                acc[c][3] = __builtin_fmaf(w, x.w, acc[c][3]);
+            }
+        }
+        if (more) {
+            store_window((t + 1) & 1u);
+#pragma unroll
+            for (int c = 0; c < CPW; ++c) { ecnt[c] = ncnt[c]; ent[c] = nent[c]; }
+        }
+        __syncthreads();
+    }
+
+    if (live) {
+        const uint32_t ho = th0 + ty, wo = tw0 + tx;
+#pragma unroll
+        for (int c = 0; c < CPW; ++c) {
+            const uint32_t co = co0 + c;
+            if (co < g.Cout) {
+                float4 out;
+                out.x = so_epilogue<ACT>(acc[c][0]); out.y = so_epilogue<ACT>(acc[c][1]);
+                out.z = so_epilogue<ACT>(acc[c][2]); out.w = so_epilogue<ACT>(acc[c][3]);
+                *reinterpret_cast<float4 *>(Y + (((size_t)co * g.H_out + ho) * g.W_out + wo) * B + bz + b4 * 4u) = out;
+            }
+        }
+    }
+}
+
+template <int CPW, int LPP>
+void window_launch_act(so_ctx *ctx, const so_conv_plan *plan, const WinArgs &a, dim3 grid, size_t lds,
+                       const float *dX, uint32_t B, const float *dBias, float *dY, int act)
+{
+#define SO_WIN_LAUNCH(A)                                                                                   \
+    conv2d_window_kernel<CPW, LPP, A><<<grid, kWinThreads, lds, ctx->stream>>>(                            \
+        plan->win.d_went, plan->win.d_cstart, a, plan->g, dX, B, dBias, dY)
+    switch (act) {
+    case SO_ACT_RELU:    SO_WIN_LAUNCH(SO_ACT_RELU); break;
+    case SO_ACT_SIGMOID: SO_WIN_LAUNCH(SO_ACT_SIGMOID); break;
+    case SO_ACT_TANH:    SO_WIN_LAUNCH(SO_ACT_TANH); break;
+    default:             SO_WIN_LAUNCH(SO_ACT_NONE); break;
+    }
+#undef SO_WIN_LAUNCH
+}
+
+// The windowed kernels use more than the default 64 KB of dynamic LDS: raise the limit of every
+// instantiation once, at plan creation (never from so_conv2d, which may run under graph capture).
+template <int CPW, int LPP>
+hipError_t window_allow_lds(int bytes)
+{
+    hipError_t e = hipSuccess;
+    const void *k[4] = {(const void *)conv2d_window_kernel<CPW, LPP, SO_ACT_NONE>, (const void *)conv2d_window_kernel<CPW, LPP, SO_ACT_RELU>,
+                        (const void *)conv2d_window_kernel<CPW, LPP, SO_ACT_SIGMOID>, (const void *)conv2d_window_kernel<CPW, LPP, SO_ACT_TANH>};
+    for (const void *f : k)
+        if (e == hipSuccess) e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    return e;
+}
+
+so_status window_configure(so_ctx *ctx)
+{
+    static bool configured = false;
+    if (configured) return SO_OK;
+    SO_HIP((window_allow_lds<4, 8>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<2, 8>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<4, 4>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<2, 4>(ctx->max_lds_bytes)));
+    configured = true;
+    return SO_OK;
+}
+
+// Launches the windowed kernel if the plan has the layout, the batch suits it and the grid
+// covers the chip; *done says whether it did.
+template <int LPP>
+so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B, const float *dBias,
+                        float *dY, int act, bool forced, bool *done)
+{
+    const so_conv_window &w = plan->win;
+    constexpr uint32_t BT = LPP * 4, PPW = 64 / LPP;
+    WinArgs a;
+    a.TH = w.TH; a.TW = w.TW; a.IH = w.IH; a.IW = w.IW; a.cc = w.cc; a.nch = w.nch; a.tiles_x = w.tiles_x;
+    a.pg = so_ceil_div(w.TH * w.TW, PPW);
+    if (a.pg == 0 || a.pg > 16) return SO_OK;
+    a.cg = 16 / a.pg;
+    a.win_f4 = w.cc * w.IH * w.IW * LPP;
+    a.r = plan->E->r;
+    if (a.win_f4 > (uint32_t)kWinMaxPerThread * kWinThreads) return SO_OK;
+    const size_t lds = 2ull * a.win_f4 * 16;
+    if (lds > (size_t)ctx->max_lds_bytes) return SO_OK;
+    const dim3 grid(w.tiles_x * w.tiles_y, so_ceil_div(plan->g.Cout, a.cg * (uint32_t)w.cpw), B / BT);
+    const uint64_t groups = (uint64_t)grid.x * grid.y * grid.z;
+    if (!forced && 4 * groups < 3 * (uint64_t)ctx->compute_units) return SO_OK;      // too few workgroups for the chip
+    if (grid.y > 65535u || grid.z > 65535u) return SO_OK;
+    if (w.cpw == 4) window_launch_act<4, LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act);
+    else window_launch_act<2, LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act);
+    *done = true;
+    return SO_OK;
+}
+
 template <int VEC>
 void conv_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B, uint64_t ncols,
                  const float *dBias, float *dY, int act)
@@ -165,6 +423,97 @@ void conv_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_
     default:             SO_CONV_LAUNCH(SO_ACT_NONE); break;
     }
 #undef SO_CONV_LAUNCH
+}
+
+
+// Chooses tile, channel chunk and channels per wave for the windowed kernel and uploads its
+// arrays.  Leaves plan->win.cc == 0 when the geometry does not suit the kernel (taps of one
+// chunk must fit the 64 lanes of a wave; a chunk must hold enough nonzeros to amortise its
+// copy; the whole output must give the chip enough workgroups at batch tile 32).
+so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32_t> &idx,
+                       const std::vector<uint32_t> &nnz, const std::vector<float> &Wd)
+{
+    const so_conv_geom &g = plan->g;
+    const so_ellpack *E = plan->E;
+    const uint32_t kHW = g.kH * g.kW;
+    if (kHW == 0 || kHW > 64 || E->r == 0 || E->total_nnz == 0) return SO_OK;
+    // Tile: at most 32 output pixels (4 pixel groups of 8 at batch tile 32); fewest tiles, then smallest window.
+    uint32_t bestTH = 0, bestTW = 0;
+    uint64_t best_tiles = ~0ull, best_win = ~0ull;
+    for (uint32_t th = 1; th <= 32 && th <= g.H_out; ++th)
+        for (uint32_t tw = 1; th * tw <= 32 && tw <= g.W_out; ++tw) {
+            const uint64_t tiles = (uint64_t)so_ceil_div(g.H_out, th) * so_ceil_div(g.W_out, tw);
+            const uint64_t win = (uint64_t)((th - 1) * g.stride_h + (g.kH - 1) * g.dil_h + 1) *
+                                 ((tw - 1) * g.stride_w + (g.kW - 1) * g.dil_w + 1);
+            if (tiles < best_tiles || (tiles == best_tiles && win < best_win)) {
+                best_tiles = tiles; best_win = win; bestTH = th; bestTW = tw;
+            }
+        }
+    if (bestTH == 0) return SO_OK;
+    so_conv_window w;
+    w.TH = bestTH; w.TW = bestTW;
+    w.IH = (w.TH - 1) * g.stride_h + (g.kH - 1) * g.dil_h + 1;
+    w.IW = (w.TW - 1) * g.stride_w + (g.kW - 1) * g.dil_w + 1;
+    w.tiles_y = so_ceil_div(g.H_out, w.TH);
+    w.tiles_x = so_ceil_div(g.W_out, w.TW);
+    if ((uint64_t)w.IH * w.IW > 4096) return SO_OK;
+    // Channel chunk: taps fit one wave, two windows of batch tile 32 fit LDS and the copy loop.
+    const uint64_t px_bytes = 32 * 4, lds_budget = (uint64_t)ctx->max_lds_bytes;
+    uint32_t cc = std::min<uint32_t>(64 / kHW, g.Cin);
+    while (cc > 0 && (2ull * cc * w.IH * w.IW * px_bytes > lds_budget ||
+                      (uint64_t)cc * w.IH * w.IW * 8 > (uint64_t)kWinMaxPerThread * kWinThreads))
+        --cc;
+    if (cc == 0) return SO_OK;
+    w.cc = cc;
+    w.nch = so_ceil_div(g.Cin, cc);
+    // Enough nonzeros per (channel, chunk) to pay for the chunk's barrier and copy.
+    if ((double)E->total_nnz / ((double)g.Cout * w.nch) < 6.0) return SO_OK;
+    if ((uint64_t)cc * g.H_in * g.W_in >= (1ull << 24)) return SO_OK;   // int32 offsets up to batch 128
+    // Channels per wave: as many as still give the chip enough workgroups (4 channel groups at batch tile 32).
+    const uint64_t tiles = (uint64_t)w.tiles_x * w.tiles_y;
+    w.cpw = 0;
+    for (int cpw : {4, 2})
+        if (tiles * so_ceil_div(g.Cout, 4u * (uint32_t)cpw) >= 3ull * (uint64_t)ctx->compute_units / 4) { w.cpw = cpw; break; }
+    if (w.cpw == 0) w.cpw = 2;
+
+    const size_t slots = (size_t)E->m * E->r;
+    std::vector<int2> went(slots, make_int2(0, 0));
+    std::vector<uint32_t> cstart((size_t)E->m * (w.nch + 1), 0);
+    for (uint32_t co = 0; co < E->m; ++co) {
+        uint32_t t = 0;
+        uint32_t *cs = &cstart[(size_t)co * (w.nch + 1)];
+        for (uint32_t j = 0; j < nnz[co]; ++j) {
+            const uint32_t k = idx[(size_t)co * E->r + j];
+            const uint32_t cin = k / kHW, kh = (k / g.kW) % g.kH, kw = k % g.kW;
+            while (t < cin / cc) cs[++t] = j;                 // slots ascend in k, hence in cin
+            const uint32_t cl = cin % cc;
+            int2 e;
+            uint32_t wb;
+            std::memcpy(&wb, &Wd[(size_t)co * E->r + j], 4);
+            e.x = (int32_t)wb;
+            e.y = (int32_t)((cl * w.IH + kh * g.dil_h) * w.IW + kw * g.dil_w);
+            went[(size_t)co * E->r + j] = e;
+        }
+        while (t < w.nch) cs[++t] = nnz[co];
+        for (uint32_t q = 0; q < w.nch; ++q)
+            if (cs[q + 1] - cs[q] > 64) return SO_OK;          // cannot happen while cc * kH * kW <= 64
+    }
+    void *d1 = nullptr, *d2 = nullptr;
+    so_status s = window_configure(ctx);
+    if (s != SO_OK) return s;
+    s = so_malloc(ctx, slots * sizeof(int2) + 16, &d1);
+    if (s == SO_OK) s = so_h2d(ctx, d1, went.data(), slots * sizeof(int2));
+    if (s == SO_OK) s = so_malloc(ctx, cstart.size() * sizeof(uint32_t), &d2);
+    if (s == SO_OK) s = so_h2d(ctx, d2, cstart.data(), cstart.size() * sizeof(uint32_t));
+    if (s != SO_OK) {
+        if (d1) (void)hipFree(d1);
+        if (d2) (void)hipFree(d2);
+        return s;
+    }
+    w.d_went = (int2 *)d1;
+    w.d_cstart = (uint32_t *)d2;
+    plan->win = w;
+    return SO_OK;
 }
 
 } // namespace
@@ -192,7 +541,8 @@ extern "C" so_status so_conv_plan_create(so_ctx *ctx, const so_ellpack *E, const
 
     const size_t slots = (size_t)E->m * E->r;
     std::vector<uint32_t> idx(slots), nnz(E->m);
-    so_status s = so_ellpack_download(ctx, E, SO_LAYOUT_ROW, nullptr, idx.data(), nnz.data());
+    std::vector<float> Wd(slots);
+    so_status s = so_ellpack_download(ctx, E, SO_LAYOUT_ROW, Wd.data(), idx.data(), nnz.data());
     if (s != SO_OK) return s;
     std::vector<int2> taps(slots, int2{0, 0});
     const uint32_t kHW = g->kH * g->kW;
@@ -219,6 +569,12 @@ extern "C" so_status so_conv_plan_create(so_ctx *ctx, const so_ellpack *E, const
         return s;
     }
     plan->d_taps = (int2 *)d;
+    s = build_window(ctx, plan, idx, nnz, Wd);
+    if (s != SO_OK) {
+        (void)hipFree(plan->d_taps);
+        delete plan;
+        return s;
+    }
     *out = plan;
     return SO_OK;
 }
@@ -228,7 +584,18 @@ extern "C" so_status so_conv_plan_free(so_ctx *ctx, so_conv_plan *plan)
     if (!plan) return SO_OK;
     if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (plan->d_taps) (void)hipFree(plan->d_taps);
+    if (plan->win.d_went) (void)hipFree(plan->win.d_went);
+    if (plan->win.d_cstart) (void)hipFree(plan->win.d_cstart);
     delete plan;
+    return SO_OK;
+}
+
+extern "C" so_status so_conv_plan_window(const so_conv_plan *plan, uint32_t out[8])
+{
+    SO_REQUIRE(plan && out, "so_conv_plan_window: null argument");
+    const so_conv_window &w = plan->win;
+    const uint32_t v[8] = {w.TH, w.TW, w.IH, w.IW, w.cc, w.nch, (uint32_t)w.cpw, 0u};
+    for (int i = 0; i < 8; ++i) out[i] = w.cc ? v[i] : 0u;
     return SO_OK;
 }
 
@@ -246,6 +613,22 @@ extern "C" so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const floa
     const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY;
     int maxvec = 4;
     if (const char *e = getenv("SPARSEOPS_CONV_VEC")) maxvec = atoi(e);
+    // The LDS-windowed kernel when the plan carries its layout and the batch splits into tiles of
+    // 32 or 16 (SPARSEOPS_CONV_WINDOW=1 forces it whenever possible, =0 forbids it: tuning and tests).
+    if (plan->win.cc != 0 && B % 16 == 0 && (align & 15) == 0 && (uint64_t)plan->win.cc * g.H_in * g.W_in * B < (1ull << 31)) {
+        const char *force = getenv("SPARSEOPS_CONV_WINDOW");
+        const bool forced = force && force[0] == '1';
+        if (!(force && force[0] == '0')) {
+            bool done = false;
+            const so_status s = (B % 32 == 0) ? window_launch<8>(ctx, plan, dX, B, dBias, dY, act, forced, &done)
+                                              : window_launch<4>(ctx, plan, dX, B, dBias, dY, act, forced, &done);
+            if (s != SO_OK) return s;
+            if (done) {
+                SO_LAUNCH_CHECK();
+                return SO_OK;
+            }
+        }
+    }
     if (maxvec >= 4 && B % 4 == 0 && (align & 15) == 0) conv_launch<4>(ctx, plan, dX, B, ncols, dBias, dY, act);
     else if (maxvec >= 2 && B % 2 == 0 && (align & 7) == 0) conv_launch<2>(ctx, plan, dX, B, ncols, dBias, dY, act);
     else conv_launch<1>(ctx, plan, dX, B, ncols, dBias, dY, act);

@@ -2,6 +2,8 @@
 the GPU against the oracle: bit-exact for everything whose arithmetic is fixed
 (conv with NONE/RELU, max, the ordered GAP sum, add, relu, transpose), 1e-6
 relative for the sigmoid/tanh library calls."""
+import os
+
 import numpy as np
 import pytest
 
@@ -13,9 +15,22 @@ import hipabi
 pytestmark = pytest.mark.gpu
 
 
-def gpu_conv(ctx, E, g, X, B, bias, act="none"):
+def gpu_conv(ctx, E, g, X, B, bias, act="none", window=None):
+    """window=True forces the LDS-windowed kernel (and requires that the plan offers it),
+    False forbids it, None leaves the library's own choice."""
     dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
     plan = ctx.conv_plan(dE, g)
+    if window is not None:
+        os.environ["SPARSEOPS_CONV_WINDOW"] = "1" if window else "0"
+        if window:
+            assert ctx.conv_plan_window(plan) is not None and B % 16 == 0
+    try:
+        return _gpu_conv(ctx, dE, plan, g, X, B, bias, act)
+    finally:
+        os.environ.pop("SPARSEOPS_CONV_WINDOW", None)
+
+
+def _gpu_conv(ctx, dE, plan, g, X, B, bias, act):
     dX, dY = ctx.array(X), ctx.empty((g.Cout, g.H_out, g.W_out, B))
     dB = ctx.array(bias) if bias is not None else None
     ctx.conv2d(plan, dX, B, dB, dY, act)
@@ -46,6 +61,41 @@ def test_conv_bit_exact(ctx, oracle, Cin, Cout, H, Wi, B, k, s, p, d):
             assert np.array_equal(gpu_conv(ctx, E, g, X, B, bias, act), oracle.conv2d_pf(as_oracle(E), og, X, B, bias, act))
     for act in ("sigmoid", "tanh"):
         assert rel_err(gpu_conv(ctx, E, g, X, B, b, act), oracle.conv2d_pf(as_oracle(E), og, X, B, b, act)) <= 1e-6
+
+
+# (Cin, Cout, H, W, B, kernel, stride, pad, dilation, sparsity): shapes the windowed kernel takes
+WINDOW_CASES = [
+    (16, 32, 28, 28, 32, (3, 3), (1, 1), (1, 1), (1, 1), .7),     # whole tiles, 3 chunks (16 = 7 + 7 + 2)
+    (9, 21, 13, 11, 32, (3, 3), (1, 1), (1, 1), (1, 1), .5),      # ragged tiles, channels and channel block
+    (16, 24, 30, 30, 16, (3, 3), (2, 2), (1, 1), (1, 1), .6),     # stride 2, batch tile 16
+    (3, 64, 32, 32, 32, (7, 7), (2, 2), (3, 3), (1, 1), .7),      # stem: one channel per chunk
+    (8, 8, 12, 12, 64, (3, 3), (1, 1), (2, 2), (2, 2), .5),       # dilation 2, two batch tiles
+    (4, 5, 10, 17, 48, (3, 2), (1, 2), (2, 0), (2, 1), .3),       # odd kernel, strides and pads; batch 48 = 3 tiles of 16
+    (2, 9, 9, 9, 32, (5, 5), (1, 1), (2, 2), (1, 1), .5),         # 5x5
+    (64, 64, 8, 8, 16, (3, 3), (1, 1), (1, 1), (1, 1), .8),       # 10 chunks, image smaller than... one tile row
+    (20, 6, 6, 6, 32, (1, 1), (1, 1), (0, 0), (1, 1), .3),        # 1x1 with enough nonzeros per chunk
+]
+
+
+@pytest.mark.parametrize("Cin,Cout,H,Wi,B,k,s,p,d,sp", WINDOW_CASES)
+def test_conv_lds_window_kernel(ctx, oracle, Cin, Cout, H, Wi, B, k, s, p, d, sp):
+    """The LDS-windowed kernel gives the gather kernel's and the oracle's bits."""
+    from oracle import conv_geom as ocg
+    rng = np.random.default_rng(Cin * 1000 + Cout * 10 + B)
+    Wc = sparse_matrix(rng, Cout, Cin * k[0] * k[1], sp)
+    Wc[Cout // 2] = 0                                      # an output channel without nonzeros
+    if Cout > 3:
+        Wc[1] = rng.standard_normal(Wc.shape[1])           # a dense one: every chunk full
+    X = rng.standard_normal((Cin, H, Wi, B)).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    E = datagen.encode_dense(Wc)
+    g, og = hipabi.conv_geom(Cin, Cout, k[0], k[1], H, Wi, s, p, d), ocg(Cin, Cout, k[0], k[1], H, Wi, s, p, d)
+    for act in ("none", "relu"):
+        for bias in (b, None):
+            Yo = oracle.conv2d_pf(as_oracle(E), og, X, B, bias, act)
+            assert np.array_equal(gpu_conv(ctx, E, g, X, B, bias, act, window=True), Yo)
+    assert np.array_equal(gpu_conv(ctx, E, g, X, B, b, "none", window=False), oracle.conv2d_pf(as_oracle(E), og, X, B, b))
+    assert rel_err(gpu_conv(ctx, E, g, X, B, b, "tanh", window=True), oracle.conv2d_pf(as_oracle(E), og, X, B, b, "tanh")) <= 1e-6
 
 
 def test_conv_reference_vectors(ctx, golden):
