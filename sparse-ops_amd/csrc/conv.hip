@@ -24,14 +24,21 @@
 
 // What the LDS-windowed kernel needs on top of the plan; built only for geometries it suits.
 // The input channels are cut into chunks of `cc`; for one chunk and one tile of TH x TW output
-// pixels the input window is IH x IW pixels.  A stored nonzero becomes {weight bits, pixel
-// offset of its tap inside the chunk's window}; cstart[co*(nch+1) + t] is the slot at which
-// chunk t begins in row co (slots are ordered by input channel, so chunks are slot ranges).
+// pixels the input window is IH x IW pixels.  A stored nonzero becomes the entry {weight bits,
+// pixel offset of its tap inside the chunk's window}.  Output channels are taken `cpw` at a
+// time (the channels one wave accumulates); the entries of such a channel group are one
+// contiguous stream in the order the wave consumes them: chunk by chunk, inside a chunk channel
+// by channel, inside a channel in slot order (slots are ordered by input channel, so a chunk is
+// a slot range).  Every (chunk, channel) run is padded to a multiple of four entries with
+// {-0.0, offset of an all-zero plane kept behind the window}: fma(-0, +0, acc) leaves any
+// accumulator as it is.
 struct so_conv_window {
     uint32_t TH = 0, TW = 0, IH = 0, IW = 0, cc = 0, nch = 0, tiles_x = 0, tiles_y = 0;
-    int cpw = 0;                  // output channels per wave: 4 or 2 (8 would spill registers)
-    int2 *d_went = nullptr;       // [Cout * r]
-    uint32_t *d_cstart = nullptr; // [Cout * (nch + 1)]
+    uint32_t groups = 0;          // ceil(Cout / cpw)
+    int cpw = 0;                  // output channels per wave
+    int2 *d_stream = nullptr;     // all groups' streams, followed by one padding quad
+    uint32_t *d_gbase = nullptr;  // [groups]: first quad (4 entries) of the group's stream
+    uint32_t *d_quads = nullptr;  // [groups * nch * cpw]: quads of (group, chunk, channel in group)
 };
 
 struct so_conv_plan {
@@ -170,35 +177,42 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
 // A workgroup of 16 waves owns a tile of TH x TW output pixels x BT batch entries and a block
 // of output channels.  It walks the input channels in chunks; a chunk's input window (halo
 // included, out-of-image pixels as zeros) is copied to LDS once and every tap of every output
-// channel of the block is then a 16-byte LDS read, about three times the rate the L1 gathers
-// of the kernel above sustain.  Lanes: LPP = BT/4 lanes per pixel (4 batch entries each), so a
-// wave covers 64/LPP pixels; the 16 waves are PG pixel groups x CG channel groups and a wave
-// accumulates CPW output channels.  The chunk's nonzeros of one output channel (at most 64)
-// sit one per lane in a register pair and are handed to the whole wave with v_readlane, so the
-// weight is a scalar operand and the tap offset a scalar addend.  Per output the multiply-adds
-// run in slot order (chunks ascend, slots ascend inside a chunk): same bits as the kernel above.
-// Windows are double-buffered: chunk t+1 is fetched into registers while chunk t is computed.
+// channel of the block is then a 16-byte LDS read, which LDS delivers at more than twice the
+// rate the L1 gathers of the kernel above sustain.  Lanes: LPP = BT/4 lanes per pixel (4 batch
+// entries each), so a wave covers 64/LPP pixels; the 16 waves are PG pixel groups x CG channel
+// groups and a wave accumulates CPW output channels.  Entries are wave-uniform: they arrive
+// through scalar loads, four at a time and one quad ahead, so the weight is a scalar operand
+// of the multiply-adds and the tap offset a scalar addend of the LDS address (handing them
+// round with v_readlane was measured at three plain VALU slots per value).  Per output the
+// multiply-adds run in slot order (chunks ascend, slots ascend inside a chunk): same bits as
+// the kernel above.  Windows are double-buffered: chunk t+1 is fetched into registers while
+// chunk t is computed.
 constexpr int kWinThreads = 1024;
 constexpr int kWinMaxPerThread = 6;   // float4 window elements a thread copies per chunk
 
 struct WinArgs {
-    uint32_t TH, TW, IH, IW, cc, nch, tiles_x, pg, cg, win_f4, r;
+    uint32_t TH, TW, IH, IW, cc, nch, tiles_x, pg, cg, groups;
+    uint32_t win_f4;    // float4 elements of one chunk's window
+    uint32_t buf_f4;    // window plus the zero plane: stride between the two buffers
 };
 
 template <int CPW, int LPP, int ACT>
 __global__ __launch_bounds__(kWinThreads)
-void conv2d_window_kernel(const int2 *__restrict__ went, const uint32_t *__restrict__ cstart, WinArgs a, so_conv_geom g,
+void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__restrict__ gbase,
+                          const uint32_t *__restrict__ quads, WinArgs a, so_conv_geom g,
                           const float *__restrict__ X, uint32_t B, const float *__restrict__ bias, float *__restrict__ Y)
 {
     extern __shared__ float4 win_lds[];
     constexpr uint32_t BT = LPP * 4, PPW = 64 / LPP, SHIFT = (LPP == 8 ? 7 : LPP == 4 ? 6 : LPP == 2 ? 5 : 4);
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t pgi = wave % a.pg, cgi = wave / a.pg;             // waves with cgi >= cg only help copying
+    const uint32_t pgi = wave % a.pg, cgi = wave / a.pg;
     const uint32_t th0 = (blockIdx.x / a.tiles_x) * a.TH, tw0 = (blockIdx.x % a.tiles_x) * a.TW;
-    const uint32_t co0 = (blockIdx.y * a.cg + cgi) * CPW;
+    const uint32_t grp = blockIdx.y * a.cg + cgi;                    // channel group of this wave
+    const uint32_t co0 = grp * CPW;
     const uint32_t bz = blockIdx.z * BT;
-    const bool computes = cgi < a.cg;
+    const bool computes = cgi < a.cg && grp < a.groups;              // the other waves only help copying
+    const uint32_t gi = computes ? grp : 0u;
 
     // this lane's output pixel and its corner inside the window
     const uint32_t pl = pgi * PPW + lane / LPP, b4 = lane % LPP;
@@ -207,7 +221,7 @@ void conv2d_window_kernel(const int2 *__restrict__ went, const uint32_t *__restr
     const uint32_t ty = pc / a.TW, tx = pc % a.TW;
     const bool live = computes && pvalid && th0 + ty < g.H_out && tw0 + tx < g.W_out;
     const uint32_t lanebase = ((ty * g.stride_h * a.IW + tx * g.stride_w) << SHIFT) + b4 * 16u;   // bytes
-    const uint32_t buf_bytes = a.win_f4 * 16u;
+    const uint32_t buf_bytes = a.buf_f4 * 16u;
 
     // window elements this thread copies: element e = tid + k*1024 is float4 (cl, ih, iw, b4)
     int32_t goff[kWinMaxPerThread];      // float offset from the chunk's first channel; -1: outside the image
@@ -242,24 +256,7 @@ void conv2d_window_kernel(const int2 *__restrict__ went, const uint32_t *__restr
     auto store_window = [&](uint32_t buf) {
 #pragma unroll
         for (int k = 0; k < kWinMaxPerThread; ++k)
-            if (gcl[k] != 0xffffffffu) win_lds[buf * a.win_f4 + tid + (uint32_t)k * kWinThreads] = xr[k];
-    };
-
-    // the chunk's nonzeros of each of this wave's output channels, one per lane
-    uint32_t ecnt[CPW], ncnt[CPW];
-    int2 ent[CPW], nent[CPW];
-    auto fetch_entries = [&](uint32_t t, uint32_t (&cnt)[CPW], int2 (&e)[CPW]) {
-#pragma unroll
-        for (int c = 0; c < CPW; ++c) {
-            const uint32_t co = co0 + c;
-            cnt[c] = 0;
-            e[c] = make_int2(0, 0);
-            if (computes && co < g.Cout) {
-                const uint32_t s0 = cstart[(size_t)co * (a.nch + 1) + t], s1 = cstart[(size_t)co * (a.nch + 1) + t + 1];
-                cnt[c] = s1 - s0;
-                if (lane < cnt[c]) e[c] = went[(size_t)co * a.r + s0 + lane];
-            }
-        }
+            if (gcl[k] != 0xffffffffu) win_lds[buf * a.buf_f4 + tid + (uint32_t)k * kWinThreads] = xr[k];
     };
 
     float acc[CPW][4];
@@ -269,56 +266,55 @@ void conv2d_window_kernel(const int2 *__restrict__ went, const uint32_t *__restr
         acc[c][0] = acc[c][1] = acc[c][2] = acc[c][3] = b0;
     }
 
+    // the all-zero plane behind each window buffer (padding entries point into it)
+    for (uint32_t i = tid; i < a.buf_f4 - a.win_f4; i += kWinThreads) {
+        win_lds[a.win_f4 + i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        win_lds[a.buf_f4 + a.win_f4 + i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     fetch_window(0);
-    fetch_entries(0, ecnt, ent);
     store_window(0);
+
+    // The wave's entry stream: one quad = 4 entries = two int4 {w0, o0, w1, o1}, {w2, o2, w3, o3}.
+    // `cur` is the quad about to be used, the next one is requested before cur is consumed; the
+    // stream ends with a padding quad, so the request after the last quad is harmless.
+    const int4 *__restrict__ sp = stream + 2 * (size_t)gbase[gi];
+    const uint32_t *__restrict__ qp = quads + (size_t)gi * a.nch * CPW;
+    int4 cur0 = sp[0], cur1 = sp[1];
+    sp += 2;
     __syncthreads();
 
     const char *lds_bytes = reinterpret_cast<const char *>(win_lds);
     for (uint32_t t = 0; t < a.nch; ++t) {
         const bool more = t + 1 < a.nch;
-        if (more) {
-            fetch_window(t + 1);
-            fetch_entries(t + 1, ncnt, nent);
-        }
+        if (more) fetch_window(t + 1);
         const uint32_t base = lanebase + (t & 1u) * buf_bytes;
+        uint32_t nq[CPW];
+#pragma unroll
+        for (int c = 0; c < CPW; ++c) nq[c] = computes ? qp[t * CPW + c] : 0u;
 #pragma unroll
         for (int c = 0; c < CPW; ++c) {
-            const uint32_t cnt = ecnt[c];
-            const int wbits = ent[c].x, offs = ent[c].y;
-            uint32_t e = 0;
-            for (; e + 4 <= cnt; e += 4) {
-                float w[4];
-                float4 x[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    w[u] = __int_as_float(__builtin_amdgcn_readlane(wbits, (int)(e + u)));
-                    const uint32_t o = (uint32_t)__builtin_amdgcn_readlane(offs, (int)(e + u));
-                    x[u] = *reinterpret_cast<const float4 *>(lds_bytes + base + (o << SHIFT));
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    acc[c][0] = __builtin_fmaf(w[u], x[u].x, acc[c][0]);
-                    acc[c][1] = __builtin_fmaf(w[u], x[u].y, acc[c][1]);
-                    acc[c][2] = __builtin_fmaf(w[u], x[u].z, acc[c][2]);
-                    acc[c][3] = __builtin_fmaf(w[u], x[u].w, acc[c][3]);
-                }
-            }
-            for (; e < cnt; ++e) {
-                const float w = __int_as_float(__builtin_amdgcn_readlane(wbits, (int)e));
-                const uint32_t o = (uint32_t)__builtin_amdgcn_readlane(offs, (int)e);
-                const float4 x = *reinterpret_cast<const float4 *>(lds_bytes + base + (o << SHIFT));
-                acc[c][0] = __builtin_fmaf(w, x.x, acc[c][0]);
-                acc[c][1] = __builtin_fmaf(w, x.y, acc[c][1]);
-                acc[c][2] = __builtin_fmaf(w, x.z, acc[c][2]);
-                acc[c][3] = __builtin_fmaf(w, x.w, acc[c][3]);
+            for (uint32_t q = 0; q < nq[c]; ++q) {
+                const int4 nxt0 = sp[0], nxt1 = sp[1];
+                sp += 2;
+                const float4 x0 = *reinterpret_cast<const float4 *>(lds_bytes + base + ((uint32_t)cur0.y << SHIFT));
+                const float4 x1 = *reinterpret_cast<const float4 *>(lds_bytes + base + ((uint32_t)cur0.w << SHIFT));
+                const float4 x2 = *reinterpret_cast<const float4 *>(lds_bytes + base + ((uint32_t)cur1.y << SHIFT));
+                const float4 x3 = *reinterpret_cast<const float4 *>(lds_bytes + base + ((uint32_t)cur1.w << SHIFT));
+                const float w0 = __int_as_float(cur0.x), w1 = __int_as_float(cur0.z);
+                const float w2 = __int_as_float(cur1.x), w3 = __int_as_float(cur1.z);
+                acc[c][0] = __builtin_fmaf(w0, x0.x, acc[c][0]); acc[c][1] = __builtin_fmaf(w0, x0.y, acc[c][1]);
+                acc[c][2] = __builtin_fmaf(w0, x0.z, acc[c][2]); acc[c][3] = __builtin_fmaf(w0, x0.w, acc[c][3]);
+                acc[c][0] = __builtin_fmaf(w1, x1.x, acc[c][0]); acc[c][1] = __builtin_fmaf(w1, x1.y, acc[c][1]);
+                acc[c][2] = __builtin_fmaf(w1, x1.z, acc[c][2]); acc[c][3] = __builtin_fmaf(w1, x1.w, acc[c][3]);
+                acc[c][0] = __builtin_fmaf(w2, x2.x, acc[c][0]); acc[c][1] = __builtin_fmaf(w2, x2.y, acc[c][1]);
+                acc[c][2] = __builtin_fmaf(w2, x2.z, acc[c][2]); acc[c][3] = __builtin_fmaf(w2, x2.w, acc[c][3]);
+                acc[c][0] = __builtin_fmaf(w3, x3.x, acc[c][0]); acc[c][1] = __builtin_fmaf(w3, x3.y, acc[c][1]);
+                acc[c][2] = __builtin_fmaf(w3, x3.z, acc[c][2]); acc[c][3] = __builtin_fmaf(w3, x3.w, acc[c][3]);
+                cur0 = nxt0;
+                cur1 = nxt1;
             }
         }
-        if (more) {
-            store_window((t + 1) & 1u);
-#pragma unroll
-            for (int c = 0; c < CPW; ++c) { ecnt[c] = ncnt[c]; ent[c] = nent[c]; }
-        }
+        if (more) store_window((t + 1) & 1u);
         __syncthreads();
     }
 
@@ -343,7 +339,8 @@ void window_launch_act(so_ctx *ctx, const so_conv_plan *plan, const WinArgs &a, 
 {
 #define SO_WIN_LAUNCH(A)                                                                                   \
     conv2d_window_kernel<CPW, LPP, A><<<grid, kWinThreads, lds, ctx->stream>>>(                            \
-        plan->win.d_went, plan->win.d_cstart, a, plan->g, dX, B, dBias, dY)
+        reinterpret_cast<const int4 *>(plan->win.d_stream), plan->win.d_gbase, plan->win.d_quads, a,       \
+        plan->g, dX, B, dBias, dY)
     switch (act) {
     case SO_ACT_RELU:    SO_WIN_LAUNCH(SO_ACT_RELU); break;
     case SO_ACT_SIGMOID: SO_WIN_LAUNCH(SO_ACT_SIGMOID); break;
@@ -370,8 +367,10 @@ so_status window_configure(so_ctx *ctx)
 {
     static bool configured = false;
     if (configured) return SO_OK;
+    SO_HIP((window_allow_lds<8, 8>(ctx->max_lds_bytes)));
     SO_HIP((window_allow_lds<4, 8>(ctx->max_lds_bytes)));
     SO_HIP((window_allow_lds<2, 8>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<8, 4>(ctx->max_lds_bytes)));
     SO_HIP((window_allow_lds<4, 4>(ctx->max_lds_bytes)));
     SO_HIP((window_allow_lds<2, 4>(ctx->max_lds_bytes)));
     configured = true;
@@ -388,19 +387,21 @@ so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, 
     constexpr uint32_t BT = LPP * 4, PPW = 64 / LPP;
     WinArgs a;
     a.TH = w.TH; a.TW = w.TW; a.IH = w.IH; a.IW = w.IW; a.cc = w.cc; a.nch = w.nch; a.tiles_x = w.tiles_x;
+    a.groups = w.groups;
     a.pg = so_ceil_div(w.TH * w.TW, PPW);
     if (a.pg == 0 || a.pg > 16) return SO_OK;
     a.cg = 16 / a.pg;
     a.win_f4 = w.cc * w.IH * w.IW * LPP;
-    a.r = plan->E->r;
+    a.buf_f4 = (w.cc + 1) * w.IH * w.IW * LPP;
     if (a.win_f4 > (uint32_t)kWinMaxPerThread * kWinThreads) return SO_OK;
-    const size_t lds = 2ull * a.win_f4 * 16;
+    const size_t lds = 2ull * a.buf_f4 * 16;
     if (lds > (size_t)ctx->max_lds_bytes) return SO_OK;
-    const dim3 grid(w.tiles_x * w.tiles_y, so_ceil_div(plan->g.Cout, a.cg * (uint32_t)w.cpw), B / BT);
-    const uint64_t groups = (uint64_t)grid.x * grid.y * grid.z;
-    if (!forced && 4 * groups < 3 * (uint64_t)ctx->compute_units) return SO_OK;      // too few workgroups for the chip
+    const dim3 grid(w.tiles_x * w.tiles_y, so_ceil_div(w.groups, a.cg), B / BT);
+    const uint64_t wgs = (uint64_t)grid.x * grid.y * grid.z;
+    if (!forced && 4 * wgs < 3 * (uint64_t)ctx->compute_units) return SO_OK;      // too few workgroups for the chip
     if (grid.y > 65535u || grid.z > 65535u) return SO_OK;
-    if (w.cpw == 4) window_launch_act<4, LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act);
+    if (w.cpw == 8) window_launch_act<8, LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act);
+    else if (w.cpw == 4) window_launch_act<4, LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act);
     else window_launch_act<2, LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act);
     *done = true;
     return SO_OK;
@@ -427,16 +428,16 @@ void conv_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_
 
 
 // Chooses tile, channel chunk and channels per wave for the windowed kernel and uploads its
-// arrays.  Leaves plan->win.cc == 0 when the geometry does not suit the kernel (taps of one
-// chunk must fit the 64 lanes of a wave; a chunk must hold enough nonzeros to amortise its
-// copy; the whole output must give the chip enough workgroups at batch tile 32).
+// arrays.  Leaves plan->win.cc == 0 when the geometry does not suit the kernel (a chunk must
+// hold enough nonzeros to amortise its copy and barrier; the whole output must give the chip
+// enough workgroups at batch tile 32).
 so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32_t> &idx,
                        const std::vector<uint32_t> &nnz, const std::vector<float> &Wd)
 {
     const so_conv_geom &g = plan->g;
     const so_ellpack *E = plan->E;
     const uint32_t kHW = g.kH * g.kW;
-    if (kHW == 0 || kHW > 64 || E->r == 0 || E->total_nnz == 0) return SO_OK;
+    if (kHW == 0 || E->r == 0 || E->total_nnz == 0) return SO_OK;
     // Tile: at most 32 output pixels (4 pixel groups of 8 at batch tile 32); fewest tiles, then smallest window.
     uint32_t bestTH = 0, bestTW = 0;
     uint64_t best_tiles = ~0ull, best_win = ~0ull;
@@ -457,61 +458,88 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     w.tiles_y = so_ceil_div(g.H_out, w.TH);
     w.tiles_x = so_ceil_div(g.W_out, w.TW);
     if ((uint64_t)w.IH * w.IW > 4096) return SO_OK;
-    // Channel chunk: taps fit one wave, two windows of batch tile 32 fit LDS and the copy loop.
+    // Channel chunk: two windows (plus their zero planes) of batch tile 32 fit LDS and the copy loop.
     const uint64_t px_bytes = 32 * 4, lds_budget = (uint64_t)ctx->max_lds_bytes;
-    uint32_t cc = std::min<uint32_t>(64 / kHW, g.Cin);
-    while (cc > 0 && (2ull * cc * w.IH * w.IW * px_bytes > lds_budget ||
+    uint32_t cc = g.Cin;
+    while (cc > 0 && (2ull * (cc + 1) * w.IH * w.IW * px_bytes > lds_budget ||
                       (uint64_t)cc * w.IH * w.IW * 8 > (uint64_t)kWinMaxPerThread * kWinThreads))
         --cc;
     if (cc == 0) return SO_OK;
-    w.cc = cc;
     w.nch = so_ceil_div(g.Cin, cc);
+    cc = so_ceil_div(g.Cin, w.nch);                 // same number of chunks, evenly filled
+    w.cc = cc;
     // Enough nonzeros per (channel, chunk) to pay for the chunk's barrier and copy.
     if ((double)E->total_nnz / ((double)g.Cout * w.nch) < 6.0) return SO_OK;
     if ((uint64_t)cc * g.H_in * g.W_in >= (1ull << 24)) return SO_OK;   // int32 offsets up to batch 128
     // Channels per wave: as many as still give the chip enough workgroups (4 channel groups at batch tile 32).
     const uint64_t tiles = (uint64_t)w.tiles_x * w.tiles_y;
-    w.cpw = 0;
-    for (int cpw : {4, 2})
-        if (tiles * so_ceil_div(g.Cout, 4u * (uint32_t)cpw) >= 3ull * (uint64_t)ctx->compute_units / 4) { w.cpw = cpw; break; }
-    if (w.cpw == 0) w.cpw = 2;
+    w.cpw = 2;
+    int cpw_max = 4;
+    if (const char *e = getenv("SPARSEOPS_CONV_CPW")) cpw_max = atoi(e);
+    for (int cpw : {8, 4, 2})
+        if (cpw <= cpw_max && tiles * so_ceil_div(g.Cout, 4u * (uint32_t)cpw) >= 3ull * (uint64_t)ctx->compute_units / 4) { w.cpw = cpw; break; }
+    const uint32_t cpw = (uint32_t)w.cpw;
+    w.groups = so_ceil_div(E->m, cpw);
 
-    const size_t slots = (size_t)E->m * E->r;
-    std::vector<int2> went(slots, make_int2(0, 0));
-    std::vector<uint32_t> cstart((size_t)E->m * (w.nch + 1), 0);
-    for (uint32_t co = 0; co < E->m; ++co) {
-        uint32_t t = 0;
-        uint32_t *cs = &cstart[(size_t)co * (w.nch + 1)];
-        for (uint32_t j = 0; j < nnz[co]; ++j) {
-            const uint32_t k = idx[(size_t)co * E->r + j];
-            const uint32_t cin = k / kHW, kh = (k / g.kW) % g.kH, kw = k % g.kW;
-            while (t < cin / cc) cs[++t] = j;                 // slots ascend in k, hence in cin
-            const uint32_t cl = cin % cc;
-            int2 e;
-            uint32_t wb;
-            std::memcpy(&wb, &Wd[(size_t)co * E->r + j], 4);
-            e.x = (int32_t)wb;
-            e.y = (int32_t)((cl * w.IH + kh * g.dil_h) * w.IW + kw * g.dil_w);
-            went[(size_t)co * E->r + j] = e;
-        }
-        while (t < w.nch) cs[++t] = nnz[co];
-        for (uint32_t q = 0; q < w.nch; ++q)
-            if (cs[q + 1] - cs[q] > 64) return SO_OK;          // cannot happen while cc * kH * kW <= 64
+    // counts per (channel, chunk), then the streams
+    std::vector<uint32_t> cnt((size_t)E->m * w.nch, 0);
+    for (uint32_t co = 0; co < E->m; ++co)
+        for (uint32_t j = 0; j < nnz[co]; ++j) ++cnt[(size_t)co * w.nch + idx[(size_t)co * E->r + j] / kHW / cc];
+    std::vector<uint32_t> gbase(w.groups), quads((size_t)w.groups * w.nch * cpw, 0);
+    uint64_t total_quads = 0;
+    for (uint32_t gi = 0; gi < w.groups; ++gi) {
+        gbase[gi] = (uint32_t)total_quads;
+        for (uint32_t t = 0; t < w.nch; ++t)
+            for (uint32_t c = 0; c < cpw; ++c) {
+                const uint32_t co = gi * cpw + c;
+                const uint32_t q = co < E->m ? (cnt[(size_t)co * w.nch + t] + 3u) / 4u : 0u;
+                quads[((size_t)gi * w.nch + t) * cpw + c] = q;
+                total_quads += q;
+            }
+        if (total_quads > 0x3fffffffull) return SO_OK;
     }
-    void *d1 = nullptr, *d2 = nullptr;
+    const float neg_zero = -0.0f;
+    uint32_t pad_bits;
+    std::memcpy(&pad_bits, &neg_zero, 4);
+    std::vector<int2> stream((size_t)(total_quads + 1) * 4, make_int2((int32_t)pad_bits, (int32_t)(cc * w.IH * w.IW)));
+    {
+        size_t pos = 0;                                            // entries written so far
+        std::vector<uint32_t> next(E->m, 0);                       // next unread slot of every row
+        for (uint32_t gi = 0; gi < w.groups; ++gi)
+            for (uint32_t t = 0; t < w.nch; ++t)
+                for (uint32_t c = 0; c < cpw; ++c) {
+                    const uint32_t co = gi * cpw + c;
+                    if (co >= E->m) continue;
+                    const uint32_t n = cnt[(size_t)co * w.nch + t];
+                    for (uint32_t e = 0; e < n; ++e) {
+                        const size_t slot = (size_t)co * E->r + next[co]++;
+                        const uint32_t k = idx[slot];
+                        const uint32_t cin = k / kHW, kh = (k / g.kW) % g.kH, kw = k % g.kW;
+                        uint32_t wb;
+                        std::memcpy(&wb, &Wd[slot], 4);
+                        stream[pos + e] = make_int2((int32_t)wb, (int32_t)(((cin - t * cc) * w.IH + kh * g.dil_h) * w.IW + kw * g.dil_w));
+                    }
+                    pos += (size_t)((n + 3u) / 4u) * 4u;
+                }
+    }
+    void *d1 = nullptr, *d2 = nullptr, *d3 = nullptr;
     so_status s = window_configure(ctx);
     if (s != SO_OK) return s;
-    s = so_malloc(ctx, slots * sizeof(int2) + 16, &d1);
-    if (s == SO_OK) s = so_h2d(ctx, d1, went.data(), slots * sizeof(int2));
-    if (s == SO_OK) s = so_malloc(ctx, cstart.size() * sizeof(uint32_t), &d2);
-    if (s == SO_OK) s = so_h2d(ctx, d2, cstart.data(), cstart.size() * sizeof(uint32_t));
+    s = so_malloc(ctx, stream.size() * sizeof(int2), &d1);
+    if (s == SO_OK) s = so_h2d(ctx, d1, stream.data(), stream.size() * sizeof(int2));
+    if (s == SO_OK) s = so_malloc(ctx, gbase.size() * sizeof(uint32_t), &d2);
+    if (s == SO_OK) s = so_h2d(ctx, d2, gbase.data(), gbase.size() * sizeof(uint32_t));
+    if (s == SO_OK) s = so_malloc(ctx, quads.size() * sizeof(uint32_t), &d3);
+    if (s == SO_OK) s = so_h2d(ctx, d3, quads.data(), quads.size() * sizeof(uint32_t));
     if (s != SO_OK) {
         if (d1) (void)hipFree(d1);
         if (d2) (void)hipFree(d2);
+        if (d3) (void)hipFree(d3);
         return s;
     }
-    w.d_went = (int2 *)d1;
-    w.d_cstart = (uint32_t *)d2;
+    w.d_stream = (int2 *)d1;
+    w.d_gbase = (uint32_t *)d2;
+    w.d_quads = (uint32_t *)d3;
     plan->win = w;
     return SO_OK;
 }
@@ -584,8 +612,9 @@ extern "C" so_status so_conv_plan_free(so_ctx *ctx, so_conv_plan *plan)
     if (!plan) return SO_OK;
     if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (plan->d_taps) (void)hipFree(plan->d_taps);
-    if (plan->win.d_went) (void)hipFree(plan->win.d_went);
-    if (plan->win.d_cstart) (void)hipFree(plan->win.d_cstart);
+    if (plan->win.d_stream) (void)hipFree(plan->win.d_stream);
+    if (plan->win.d_gbase) (void)hipFree(plan->win.d_gbase);
+    if (plan->win.d_quads) (void)hipFree(plan->win.d_quads);
     delete plan;
     return SO_OK;
 }
