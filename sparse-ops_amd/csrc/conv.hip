@@ -180,7 +180,9 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
 // channel of the block is then a 16-byte LDS read, which LDS delivers at more than twice the
 // rate the L1 gathers of the kernel above sustain.  Lanes: LPP = BT/4 lanes per pixel (4 batch
 // entries each), so a wave covers 64/LPP pixels; the 16 waves are PG pixel groups x CG channel
-// groups and a wave accumulates CPW output channels.  Entries are wave-uniform: they arrive
+// groups and a wave accumulates CPW output channels.  The batch tile is 16 (LPP = 4): measured
+// against 32 and 8 it was the fastest on every layer of the ResNet-18-shaped stack, because the
+// smaller window lets a chunk hold twice the channels (longer runs per channel, half the barriers).  Entries are wave-uniform: they arrive
 // through scalar loads, four at a time and one quad ahead, so the weight is a scalar operand
 // of the multiply-adds and the tap offset a scalar addend of the LDS address (handing them
 // round with v_readlane was measured at three plain VALU slots per value).  Per output the
@@ -189,11 +191,14 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
 // chunk t is computed.
 constexpr int kWinThreads = 1024;
 constexpr int kWinMaxPerThread = 6;   // float4 window elements a thread copies per chunk
+constexpr uint32_t kWinLPP = 4;       // lanes per pixel
+constexpr uint32_t kWinBT = 4 * kWinLPP;   // batch tile
 
 struct WinArgs {
     uint32_t TH, TW, IH, IW, cc, nch, tiles_x, pg, cg, groups;
     uint32_t win_f4;    // float4 elements of one chunk's window
     uint32_t buf_f4;    // window plus the zero plane: stride between the two buffers
+    uint32_t nbuf;      // 2: double-buffered windows; 1: a single chunk, nothing to overlap
 };
 
 template <int CPW, int LPP, int ACT>
@@ -269,7 +274,7 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
     // the all-zero plane behind each window buffer (padding entries point into it)
     for (uint32_t i = tid; i < a.buf_f4 - a.win_f4; i += kWinThreads) {
         win_lds[a.win_f4 + i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        win_lds[a.buf_f4 + a.win_f4 + i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (a.nbuf == 2) win_lds[a.buf_f4 + a.win_f4 + i] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
     fetch_window(0);
     store_window(0);
@@ -287,7 +292,8 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
     for (uint32_t t = 0; t < a.nch; ++t) {
         const bool more = t + 1 < a.nch;
         if (more) fetch_window(t + 1);
-        const uint32_t base = lanebase + (t & 1u) * buf_bytes;
+        const uint32_t cur_buf = a.nbuf == 2 ? (t & 1u) : 0u;
+        const uint32_t base = lanebase + cur_buf * buf_bytes;
         uint32_t nq[CPW];
 #pragma unroll
         for (int c = 0; c < CPW; ++c) nq[c] = computes ? qp[t * CPW + c] : 0u;
@@ -314,8 +320,14 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
                 cur1 = nxt1;
             }
         }
-        if (more) store_window((t + 1) & 1u);
-        __syncthreads();
+        if (a.nbuf == 2) {
+            if (more) store_window(cur_buf ^ 1u);
+            __syncthreads();
+        } else {
+            __syncthreads();                       // every wave has finished reading the only buffer
+            if (more) store_window(0);
+            __syncthreads();
+        }
     }
 
     if (live) {
@@ -367,42 +379,47 @@ so_status window_configure(so_ctx *ctx)
 {
     static bool configured = false;
     if (configured) return SO_OK;
-    SO_HIP((window_allow_lds<8, 8>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<4, 8>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<2, 8>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<8, 4>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<4, 4>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<2, 4>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<8, kWinLPP>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<4, kWinLPP>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<2, kWinLPP>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<1, kWinLPP>(ctx->max_lds_bytes)));
     configured = true;
     return SO_OK;
 }
 
+// Workgroups the windowed kernel launches for batch B with `cpw` channels per wave.
+uint64_t window_workgroups(const so_conv_window &w, uint32_t cout, uint32_t cpw, uint32_t B)
+{
+    const uint32_t pg = so_ceil_div(w.TH * w.TW, 64u / kWinLPP), cg = 16u / pg;
+    return (uint64_t)w.tiles_x * w.tiles_y * so_ceil_div(so_ceil_div(cout, cpw), cg) * (B / kWinBT);
+}
+
 // Launches the windowed kernel if the plan has the layout, the batch suits it and the grid
 // covers the chip; *done says whether it did.
-template <int LPP>
 so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B, const float *dBias,
                         float *dY, int act, bool forced, bool *done)
 {
     const so_conv_window &w = plan->win;
-    constexpr uint32_t BT = LPP * 4, PPW = 64 / LPP;
+    constexpr uint32_t PPW = 64 / kWinLPP;
     WinArgs a;
     a.TH = w.TH; a.TW = w.TW; a.IH = w.IH; a.IW = w.IW; a.cc = w.cc; a.nch = w.nch; a.tiles_x = w.tiles_x;
     a.groups = w.groups;
     a.pg = so_ceil_div(w.TH * w.TW, PPW);
-    if (a.pg == 0 || a.pg > 16) return SO_OK;
     a.cg = 16 / a.pg;
-    a.win_f4 = w.cc * w.IH * w.IW * LPP;
-    a.buf_f4 = (w.cc + 1) * w.IH * w.IW * LPP;
-    if (a.win_f4 > (uint32_t)kWinMaxPerThread * kWinThreads) return SO_OK;
-    const size_t lds = 2ull * a.buf_f4 * 16;
-    if (lds > (size_t)ctx->max_lds_bytes) return SO_OK;
-    const dim3 grid(w.tiles_x * w.tiles_y, so_ceil_div(w.groups, a.cg), B / BT);
+    a.win_f4 = w.cc * w.IH * w.IW * kWinLPP;
+    a.buf_f4 = (w.cc + 1) * w.IH * w.IW * kWinLPP;
+    a.nbuf = w.nch > 1 ? 2u : 1u;
+    const size_t lds = (size_t)a.nbuf * a.buf_f4 * 16;
+    const dim3 grid(w.tiles_x * w.tiles_y, so_ceil_div(w.groups, a.cg), B / kWinBT);
     const uint64_t wgs = (uint64_t)grid.x * grid.y * grid.z;
-    if (!forced && 4 * wgs < 3 * (uint64_t)ctx->compute_units) return SO_OK;      // too few workgroups for the chip
+    if (!forced && 2 * wgs < (uint64_t)ctx->compute_units) return SO_OK;      // too few workgroups for the chip
     if (grid.y > 65535u || grid.z > 65535u) return SO_OK;
-    if (w.cpw == 8) window_launch_act<8, LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act);
-    else if (w.cpw == 4) window_launch_act<4, LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act);
-    else window_launch_act<2, LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act);
+    switch (w.cpw) {
+    case 8:  window_launch_act<8, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act); break;
+    case 4:  window_launch_act<4, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act); break;
+    case 2:  window_launch_act<2, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act); break;
+    default: window_launch_act<1, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act); break;
+    }
     *done = true;
     return SO_OK;
 }
@@ -438,7 +455,7 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     const so_ellpack *E = plan->E;
     const uint32_t kHW = g.kH * g.kW;
     if (kHW == 0 || E->r == 0 || E->total_nnz == 0) return SO_OK;
-    // Tile: at most 32 output pixels (4 pixel groups of 8 at batch tile 32); fewest tiles, then smallest window.
+    // Tile: at most 32 output pixels (2 pixel groups of 16); fewest tiles, then smallest window.
     uint32_t bestTH = 0, bestTW = 0;
     uint64_t best_tiles = ~0ull, best_win = ~0ull;
     for (uint32_t th = 1; th <= 32 && th <= g.H_out; ++th)
@@ -458,26 +475,35 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     w.tiles_y = so_ceil_div(g.H_out, w.TH);
     w.tiles_x = so_ceil_div(g.W_out, w.TW);
     if ((uint64_t)w.IH * w.IW > 4096) return SO_OK;
-    // Channel chunk: two windows (plus their zero planes) of batch tile 32 fit LDS and the copy loop.
-    const uint64_t px_bytes = 32 * 4, lds_budget = (uint64_t)ctx->max_lds_bytes;
+    // Channel chunk: two windows (plus their zero planes) fit LDS, one window fits the copy loop.
+    const uint64_t px_bytes = kWinBT * 4, lds_budget = (uint64_t)ctx->max_lds_bytes;
     uint32_t cc = g.Cin;
-    while (cc > 0 && (2ull * (cc + 1) * w.IH * w.IW * px_bytes > lds_budget ||
-                      (uint64_t)cc * w.IH * w.IW * 8 > (uint64_t)kWinMaxPerThread * kWinThreads))
+    while (cc > 0 && ((cc < g.Cin ? 2ull : 1ull) * (cc + 1) * w.IH * w.IW * px_bytes > lds_budget ||
+                      (uint64_t)cc * w.IH * w.IW * kWinLPP > (uint64_t)kWinMaxPerThread * kWinThreads))
         --cc;
     if (cc == 0) return SO_OK;
     w.nch = so_ceil_div(g.Cin, cc);
     cc = so_ceil_div(g.Cin, w.nch);                 // same number of chunks, evenly filled
     w.cc = cc;
     // Enough nonzeros per (channel, chunk) to pay for the chunk's barrier and copy.
-    if ((double)E->total_nnz / ((double)g.Cout * w.nch) < 6.0) return SO_OK;
+    const double nnz_avg = (double)E->total_nnz / (double)g.Cout;
+    const double run = nnz_avg / w.nch;
+    if (run < 6.0) return SO_OK;
     if ((uint64_t)cc * g.H_in * g.W_in >= (1ull << 24)) return SO_OK;   // int32 offsets up to batch 128
-    // Channels per wave: as many as still give the chip enough workgroups (4 channel groups at batch tile 32).
-    const uint64_t tiles = (uint64_t)w.tiles_x * w.tiles_y;
-    w.cpw = 2;
-    int cpw_max = 4;
+    // Channels per wave.  Cost of a layer ~ rounds of workgroups over the chip x channels per wave x
+    // (fixed + per-wave share of the chunk overhead + per-run overhead); constants fitted on MI355X
+    // to the 3x3 layers of a ResNet-18-shaped stack at batch 32.
+    w.cpw = 1;
+    int cpw_max = 8;
     if (const char *e = getenv("SPARSEOPS_CONV_CPW")) cpw_max = atoi(e);
-    for (int cpw : {8, 4, 2})
-        if (cpw <= cpw_max && tiles * so_ceil_div(g.Cout, 4u * (uint32_t)cpw) >= 3ull * (uint64_t)ctx->compute_units / 4) { w.cpw = cpw; break; }
+    double best_cost = 0.0;
+    for (int cpw : {8, 4, 2, 1}) {
+        if (cpw > cpw_max && cpw != 1) continue;
+        const uint64_t wgs = window_workgroups(w, g.Cout, (uint32_t)cpw, 32);
+        const double rounds = (double)so_ceil_div((uint32_t)std::min<uint64_t>(wgs, 1u << 30), (uint32_t)ctx->compute_units);
+        const double cost = rounds * cpw * (6.5 + 10.0 / cpw + 29.0 / run);
+        if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; w.cpw = cpw; }
+    }
     const uint32_t cpw = (uint32_t)w.cpw;
     w.groups = so_ceil_div(E->m, cpw);
 
@@ -642,15 +668,14 @@ extern "C" so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const floa
     const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY;
     int maxvec = 4;
     if (const char *e = getenv("SPARSEOPS_CONV_VEC")) maxvec = atoi(e);
-    // The LDS-windowed kernel when the plan carries its layout and the batch splits into tiles of
-    // 32 or 16 (SPARSEOPS_CONV_WINDOW=1 forces it whenever possible, =0 forbids it: tuning and tests).
-    if (plan->win.cc != 0 && B % 16 == 0 && (align & 15) == 0 && (uint64_t)plan->win.cc * g.H_in * g.W_in * B < (1ull << 31)) {
+    // The LDS-windowed kernel when the plan carries its layout and the batch splits into tiles of 16
+    // (SPARSEOPS_CONV_WINDOW=1 forces it whenever possible, =0 forbids it: tuning and tests).
+    if (plan->win.cc != 0 && B % kWinBT == 0 && (align & 15) == 0 && (uint64_t)plan->win.cc * g.H_in * g.W_in * B < (1ull << 31)) {
         const char *force = getenv("SPARSEOPS_CONV_WINDOW");
         const bool forced = force && force[0] == '1';
         if (!(force && force[0] == '0')) {
             bool done = false;
-            const so_status s = (B % 32 == 0) ? window_launch<8>(ctx, plan, dX, B, dBias, dY, act, forced, &done)
-                                              : window_launch<4>(ctx, plan, dX, B, dBias, dY, act, forced, &done);
+            const so_status s = window_launch(ctx, plan, dX, B, dBias, dY, act, forced, &done);
             if (s != SO_OK) return s;
             if (done) {
                 SO_LAUNCH_CHECK();
