@@ -166,6 +166,13 @@ so_status so_conv_plan_window(const so_conv_plan *plan, uint32_t out[8]);
  * dY is [Cout][H_out][W_out][B]; dBias may be NULL. */
 so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B,
                     const float *dBias, float *dY, int act);
+/* The same convolution followed by the residual applyAdd (src/layers/add.cpp:9-76) and
+ * then the activation, in one pass: dY = act((conv(dX) + bias) + dResidual).  The sum is
+ * the fp32 addition applyAdd performs on the stored convolution output, so the result
+ * has the same bits as the three separate layers.  dResidual is [Cout][H_out][W_out][B]
+ * and must not alias dY. */
+so_status so_conv2d_add(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B,
+                        const float *dBias, const float *dResidual, float *dY, int act);
 
 /* applyMaxPool / applyGlobalAveragePool (src/layers/pool.cpp:28-101, 103-154)
  * on [C][H][W][B]; GAP writes [C][B]. */

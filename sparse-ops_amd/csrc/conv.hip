@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kChannelsPerGroup * 64)
 void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict__ taps,
                             const uint32_t *__restrict__ nnz, uint32_t r, so_conv_geom g,
                             const float *__restrict__ X, uint32_t B, uint64_t ncols,
-                            const float *__restrict__ bias, float *__restrict__ Y)
+                            const float *__restrict__ bias, const float *__restrict__ resid, float *__restrict__ Y)
 {
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t co = __builtin_amdgcn_readfirstlane(blockIdx.y * kChannelsPerGroup + (threadIdx.x >> 6));
@@ -160,6 +160,12 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
     }
     if (live) {
         using T = typename ConvVec<VEC>::type;
+        if (resid) {                     // the residual Add that follows the convolution: conv + skip, then the activation
+            float rv[VEC];
+            conv_load<VEC>(resid + (size_t)co * ncols + q, rv);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[v] += rv[v];
+        }
         T out;
         if constexpr (VEC == 1) { out = so_epilogue<ACT>(acc[0]); }
         if constexpr (VEC == 2) { out.x = so_epilogue<ACT>(acc[0]); out.y = so_epilogue<ACT>(acc[1]); }
@@ -205,7 +211,8 @@ template <int CPW, int LPP, int ACT>
 __global__ __launch_bounds__(kWinThreads)
 void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__restrict__ gbase,
                           const uint32_t *__restrict__ quads, WinArgs a, so_conv_geom g,
-                          const float *__restrict__ X, uint32_t B, const float *__restrict__ bias, float *__restrict__ Y)
+                          const float *__restrict__ X, uint32_t B, const float *__restrict__ bias,
+                          const float *__restrict__ resid, float *__restrict__ Y)
 {
     extern __shared__ float4 win_lds[];
     constexpr uint32_t BT = LPP * 4, PPW = 64 / LPP, SHIFT = (LPP == 8 ? 7 : LPP == 4 ? 6 : LPP == 2 ? 5 : 4);
@@ -336,10 +343,15 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
         for (int c = 0; c < CPW; ++c) {
             const uint32_t co = co0 + c;
             if (co < g.Cout) {
+                const size_t at = (((size_t)co * g.H_out + ho) * g.W_out + wo) * B + bz + b4 * 4u;
+                if (resid) {             // conv + skip, then the activation
+                    const float4 rv = *reinterpret_cast<const float4 *>(resid + at);
+                    acc[c][0] += rv.x; acc[c][1] += rv.y; acc[c][2] += rv.z; acc[c][3] += rv.w;
+                }
                 float4 out;
                 out.x = so_epilogue<ACT>(acc[c][0]); out.y = so_epilogue<ACT>(acc[c][1]);
                 out.z = so_epilogue<ACT>(acc[c][2]); out.w = so_epilogue<ACT>(acc[c][3]);
-                *reinterpret_cast<float4 *>(Y + (((size_t)co * g.H_out + ho) * g.W_out + wo) * B + bz + b4 * 4u) = out;
+                *reinterpret_cast<float4 *>(Y + at) = out;
             }
         }
     }
@@ -347,12 +359,12 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
 
 template <int CPW, int LPP>
 void window_launch_act(so_ctx *ctx, const so_conv_plan *plan, const WinArgs &a, dim3 grid, size_t lds,
-                       const float *dX, uint32_t B, const float *dBias, float *dY, int act)
+                       const float *dX, uint32_t B, const float *dBias, const float *dResid, float *dY, int act)
 {
 #define SO_WIN_LAUNCH(A)                                                                                   \
     conv2d_window_kernel<CPW, LPP, A><<<grid, kWinThreads, lds, ctx->stream>>>(                            \
         reinterpret_cast<const int4 *>(plan->win.d_stream), plan->win.d_gbase, plan->win.d_quads, a,       \
-        plan->g, dX, B, dBias, dY)
+        plan->g, dX, B, dBias, dResid, dY)
     switch (act) {
     case SO_ACT_RELU:    SO_WIN_LAUNCH(SO_ACT_RELU); break;
     case SO_ACT_SIGMOID: SO_WIN_LAUNCH(SO_ACT_SIGMOID); break;
@@ -397,7 +409,7 @@ uint64_t window_workgroups(const so_conv_window &w, uint32_t cout, uint32_t cpw,
 // Launches the windowed kernel if the plan has the layout, the batch suits it and the grid
 // covers the chip; *done says whether it did.
 so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B, const float *dBias,
-                        float *dY, int act, bool forced, bool *done)
+                        const float *dResid, float *dY, int act, bool forced, bool *done)
 {
     const so_conv_window &w = plan->win;
     constexpr uint32_t PPW = 64 / kWinLPP;
@@ -415,10 +427,10 @@ so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, 
     if (!forced && 2 * wgs < (uint64_t)ctx->compute_units) return SO_OK;      // too few workgroups for the chip
     if (grid.y > 65535u || grid.z > 65535u) return SO_OK;
     switch (w.cpw) {
-    case 8:  window_launch_act<8, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act); break;
-    case 4:  window_launch_act<4, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act); break;
-    case 2:  window_launch_act<2, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act); break;
-    default: window_launch_act<1, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dY, act); break;
+    case 8:  window_launch_act<8, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
+    case 4:  window_launch_act<4, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
+    case 2:  window_launch_act<2, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
+    default: window_launch_act<1, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
     }
     *done = true;
     return SO_OK;
@@ -426,14 +438,14 @@ so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, 
 
 template <int VEC>
 void conv_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B, uint64_t ncols,
-                 const float *dBias, float *dY, int act)
+                 const float *dBias, const float *dResid, float *dY, int act)
 {
     const so_conv_geom &g = plan->g;
     const so_ellpack *E = plan->E;
     const dim3 grid((uint32_t)((ncols + 64ull * VEC - 1) / (64ull * VEC)), so_ceil_div(g.Cout, kChannelsPerGroup));
 #define SO_CONV_LAUNCH(A)                                                                          \
     conv2d_implicit_kernel<VEC, A><<<grid, kChannelsPerGroup * 64, 0, ctx->stream>>>(              \
-        E->d_Wd, plan->d_taps, E->d_nnz, E->r, g, dX, B, ncols, dBias, dY)
+        E->d_Wd, plan->d_taps, E->d_nnz, E->r, g, dX, B, ncols, dBias, dResid, dY)
     switch (act) {
     case SO_ACT_RELU:    SO_CONV_LAUNCH(SO_ACT_RELU); break;
     case SO_ACT_SIGMOID: SO_CONV_LAUNCH(SO_ACT_SIGMOID); break;
@@ -654,8 +666,8 @@ extern "C" so_status so_conv_plan_window(const so_conv_plan *plan, uint32_t out[
     return SO_OK;
 }
 
-extern "C" so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B,
-                               const float *dBias, float *dY, int act)
+static so_status conv2d_dispatch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B,
+                                 const float *dBias, const float *dResid, float *dY, int act)
 {
     SO_REQUIRE(ctx && plan, "so_conv2d: null argument");
     SO_REQUIRE(act >= SO_ACT_NONE && act <= SO_ACT_TANH, "so_conv2d: unknown activation %d", act);
@@ -665,7 +677,7 @@ extern "C" so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const floa
     SO_REQUIRE(dX && dY, "so_conv2d: null tensor");
     SO_REQUIRE((ncols + 63) / 64 < (1ull << 31), "so_conv2d: output plane too large");
     // Batch entries per lane: as many as divide B and keep 16/8-byte alignment.
-    const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY;
+    const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY | (uintptr_t)dResid;
     int maxvec = 4;
     if (const char *e = getenv("SPARSEOPS_CONV_VEC")) maxvec = atoi(e);
     // The LDS-windowed kernel when the plan carries its layout and the batch splits into tiles of 16
@@ -675,7 +687,7 @@ extern "C" so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const floa
         const bool forced = force && force[0] == '1';
         if (!(force && force[0] == '0')) {
             bool done = false;
-            const so_status s = window_launch(ctx, plan, dX, B, dBias, dY, act, forced, &done);
+            const so_status s = window_launch(ctx, plan, dX, B, dBias, dResid, dY, act, forced, &done);
             if (s != SO_OK) return s;
             if (done) {
                 SO_LAUNCH_CHECK();
@@ -683,9 +695,23 @@ extern "C" so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const floa
             }
         }
     }
-    if (maxvec >= 4 && B % 4 == 0 && (align & 15) == 0) conv_launch<4>(ctx, plan, dX, B, ncols, dBias, dY, act);
-    else if (maxvec >= 2 && B % 2 == 0 && (align & 7) == 0) conv_launch<2>(ctx, plan, dX, B, ncols, dBias, dY, act);
-    else conv_launch<1>(ctx, plan, dX, B, ncols, dBias, dY, act);
+    if (maxvec >= 4 && B % 4 == 0 && (align & 15) == 0) conv_launch<4>(ctx, plan, dX, B, ncols, dBias, dResid, dY, act);
+    else if (maxvec >= 2 && B % 2 == 0 && (align & 7) == 0) conv_launch<2>(ctx, plan, dX, B, ncols, dBias, dResid, dY, act);
+    else conv_launch<1>(ctx, plan, dX, B, ncols, dBias, dResid, dY, act);
     SO_LAUNCH_CHECK();
     return SO_OK;
+}
+
+extern "C" so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B,
+                               const float *dBias, float *dY, int act)
+{
+    return conv2d_dispatch(ctx, plan, dX, B, dBias, nullptr, dY, act);
+}
+
+extern "C" so_status so_conv2d_add(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B,
+                                   const float *dBias, const float *dResidual, float *dY, int act)
+{
+    SO_REQUIRE(dResidual, "so_conv2d_add: null residual");
+    SO_REQUIRE(dResidual != dY, "so_conv2d_add: the residual must not alias the output");
+    return conv2d_dispatch(ctx, plan, dX, B, dBias, dResidual, dY, act);
 }

@@ -19,7 +19,7 @@ LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS, LAYOUT_TILED = 1, 2, 4, 8
 SYMBOLS = (
     "so_device_count so_init so_destroy so_last_error so_device_info so_malloc so_free so_h2d so_d2h "
     "so_d2d so_fill_zero so_sync so_timer_begin so_timer_end so_ellpack_upload so_ellpack_free "
-    "so_ellpack_dims so_ellpack_download so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window "
+    "so_ellpack_dims so_ellpack_download so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv2d_add "
     "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_graph_begin so_graph_end "
     "so_graph_launch so_graph_free").split()
 
@@ -81,6 +81,7 @@ def load_library(path=None):
         "so_conv_plan_free": [_vp, _vp],
         "so_conv_plan_window": [_vp, ct.POINTER(ct.c_uint32)],
         "so_conv2d": [_vp, _vp, _vp, _u32, _vp, _vp, ct.c_int],
+        "so_conv2d_add": [_vp, _vp, _vp, ct.c_uint32, _vp, _vp, _vp, ct.c_int],
         "so_maxpool": [_vp, ct.POINTER(PoolGeom), _vp, _u32, _vp],
         "so_gap": [_vp, _u32, _u32, _u32, _vp, _u32, _vp],
         "so_add": [_vp, _vp, _vp, ct.c_size_t, _vp],
@@ -219,8 +220,11 @@ class Context:
     def conv_plan_free(self, plan):
         self.lib.so_conv_plan_free(self.h, plan)
 
-    def conv2d(self, plan, dX, B, dBias, dY, act="none"):
-        self._ck(self.lib.so_conv2d(self.h, plan, dX.ptr, B, dBias.ptr if dBias else None, dY.ptr, ACT[act]))
+    def conv2d(self, plan, dX, B, dBias, dY, act="none", residual=None):
+        if residual is None:
+            self._ck(self.lib.so_conv2d(self.h, plan, dX.ptr, B, dBias.ptr if dBias else None, dY.ptr, ACT[act]))
+        else:
+            self._ck(self.lib.so_conv2d_add(self.h, plan, dX.ptr, B, dBias.ptr if dBias else None, residual.ptr, dY.ptr, ACT[act]))
 
     def maxpool(self, C, H, W, k, s, pad, dX, B, dY):
         Ho = (H + 2 * pad[0] - k[0]) // s[0] + 1

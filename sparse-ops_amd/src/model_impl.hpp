@@ -32,6 +32,7 @@ struct LayerPlan {
     std::size_t bias_offset = 0;
     bool has_bias = false;
     int act = SO_ACT_NONE;      // fused epilogue, or the activation of an Act layer
+    bool residual = false;      // Conv: in1 is added to the convolution before the activation
 
     // pools
     so_pool_geom pg{};

@@ -55,7 +55,10 @@ void SparseOnnxModel::Impl::enqueue_layers(const float *in, float *out) const
             check(so_matmul(ctx, L.dE, src(L.in0), B, bias, dst(L.out), L.act), "so_matmul");
             break;
         case Op::Conv:
-            check(so_conv2d(ctx, L.conv, src(L.in0), B, bias, dst(L.out), L.act), "so_conv2d");
+            if (L.residual)
+                check(so_conv2d_add(ctx, L.conv, src(L.in0), B, bias, src(L.in1), dst(L.out), L.act), "so_conv2d_add");
+            else
+                check(so_conv2d(ctx, L.conv, src(L.in0), B, bias, dst(L.out), L.act), "so_conv2d");
             break;
         case Op::Act:
             check(so_act(ctx, L.act, src(L.in0), L.out_features * B, dst(L.out)), "so_act");

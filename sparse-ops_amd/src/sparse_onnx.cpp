@@ -363,21 +363,44 @@ SparseOnnxModel::SparseOnnxModel(const std::string &onnx_path) : impl_(new Impl(
     M.out_features = features_of(out_shape);
     M.output_dims = out_shape;
 
-    // Fuse an activation into the producing MatMul/Conv when nothing else reads
-    // the intermediate (src/sparse_onnx.cpp:573-620, extended to Sigmoid/Tanh).
+    // Fuse into the producing MatMul/Conv, when nothing else reads the intermediate:
+    //  * a following activation (src/sparse_onnx.cpp:573-620, extended to Sigmoid/Tanh);
+    //  * for Conv, a following residual Add whose other operand already exists when the
+    //    convolution runs, and then the activation after that Add (the tail of a ResNet
+    //    basic block: conv -> add(skip) -> relu becomes one launch, same arithmetic).
     {
         std::unordered_map<std::string, int> uses;
         for (const auto &p : pend)
             for (const auto &i : p.inputs) uses[i]++;
         uses[M.output_name]++;
+        auto produced_before = [&](const std::string &t, std::size_t layer) {
+            if (t == M.input_name) return true;
+            for (std::size_t k = 0; k < layer; ++k)
+                if (pend[k].output == t) return true;
+            return false;
+        };
         for (std::size_t i = 0; i + 1 < pend.size();) {
             Pending &A = pend[i], &Bn = pend[i + 1];
-            const bool fusable = (A.plan.op == Op::MatMul || A.plan.op == Op::Conv) && A.plan.act == SO_ACT_NONE &&
-                                 Bn.plan.op == Op::Act && Bn.inputs[0] == A.output && uses[A.output] == 1;
-            if (!fusable) { ++i; continue; }
-            A.plan.act = Bn.plan.act;
-            A.output = Bn.output;
-            pend.erase(pend.begin() + long(i) + 1);
+            const bool producer = A.plan.op == Op::MatMul || A.plan.op == Op::Conv;
+            if (producer && A.plan.act == SO_ACT_NONE && Bn.plan.op == Op::Act && Bn.inputs[0] == A.output &&
+                uses[A.output] == 1) {
+                A.plan.act = Bn.plan.act;
+                A.output = Bn.output;
+                pend.erase(pend.begin() + long(i) + 1);
+                continue;
+            }
+            if (A.plan.op == Op::Conv && A.plan.act == SO_ACT_NONE && !A.plan.residual && Bn.plan.op == Op::Add &&
+                uses[A.output] == 1 && (Bn.inputs[0] == A.output) != (Bn.inputs[1] == A.output)) {
+                const std::string skip = Bn.inputs[0] == A.output ? Bn.inputs[1] : Bn.inputs[0];
+                if (produced_before(skip, i)) {
+                    A.plan.residual = true;
+                    A.inputs.push_back(skip);
+                    A.output = Bn.output;
+                    pend.erase(pend.begin() + long(i) + 1);
+                    continue;                       // look at the same layer again: an activation may follow
+                }
+            }
+            ++i;
         }
     }
 
@@ -481,6 +504,7 @@ std::vector<std::string> SparseOnnxModel::describe() const
             for (uint32_t c : L.E->nnz) nnz += c;
             s += " " + std::to_string(L.E->m) + "x" + std::to_string(L.E->n) + " r=" + std::to_string(L.E->r) +
                  " nnz=" + std::to_string(nnz) + " act=" + act_name(L.act) + " bias=" + (L.has_bias ? "1" : "0");
+            if (L.residual) s += " +residual";
         } else if (L.op == Op::Act) {
             s += std::string(" act=") + act_name(L.act);
         }

@@ -15,7 +15,7 @@ import hipabi
 pytestmark = pytest.mark.gpu
 
 
-def gpu_conv(ctx, E, g, X, B, bias, act="none", window=None):
+def gpu_conv(ctx, E, g, X, B, bias, act="none", window=None, residual=None):
     """window=True forces the LDS-windowed kernel (and requires that the plan offers it),
     False forbids it, None leaves the library's own choice."""
     dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
@@ -25,18 +25,22 @@ def gpu_conv(ctx, E, g, X, B, bias, act="none", window=None):
         if window:
             assert ctx.conv_plan_window(plan) is not None and B % 16 == 0
     try:
-        return _gpu_conv(ctx, dE, plan, g, X, B, bias, act)
+        return _gpu_conv(ctx, dE, plan, g, X, B, bias, act, residual)
     finally:
         os.environ.pop("SPARSEOPS_CONV_WINDOW", None)
 
 
-def _gpu_conv(ctx, dE, plan, g, X, B, bias, act):
+def _gpu_conv(ctx, dE, plan, g, X, B, bias, act, residual=None):
     dX, dY = ctx.array(X), ctx.empty((g.Cout, g.H_out, g.W_out, B))
     dB = ctx.array(bias) if bias is not None else None
-    ctx.conv2d(plan, dX, B, dB, dY, act)
+    dR = ctx.array(residual) if residual is not None else None
+    ctx.conv2d(plan, dX, B, dB, dY, act, residual=dR)
     Y = dY.download()
     ctx.conv_plan_free(plan)
     dE.free()
+    for a in (dX, dY, dB, dR):
+        if a is not None:
+            a.free()
     return Y
 
 
@@ -96,6 +100,27 @@ def test_conv_lds_window_kernel(ctx, oracle, Cin, Cout, H, Wi, B, k, s, p, d, sp
             assert np.array_equal(gpu_conv(ctx, E, g, X, B, bias, act, window=True), Yo)
     assert np.array_equal(gpu_conv(ctx, E, g, X, B, b, "none", window=False), oracle.conv2d_pf(as_oracle(E), og, X, B, b))
     assert rel_err(gpu_conv(ctx, E, g, X, B, b, "tanh", window=True), oracle.conv2d_pf(as_oracle(E), og, X, B, b, "tanh")) <= 1e-6
+
+
+@pytest.mark.parametrize("B,window", [(3, False), (4, False), (32, False), (32, True), (16, True)])
+def test_conv_with_fused_residual_add(ctx, oracle, B, window):
+    """so_conv2d_add == conv, then the reference's Add, then the activation: same bits as
+    the three layers one after the other, in both convolution kernels."""
+    from oracle import conv_geom as ocg
+    rng = np.random.default_rng(B)
+    Cin, Cout, H, Wi, k = 12, 10, 9, 13, (3, 3)
+    Wc = sparse_matrix(rng, Cout, Cin * 9, .6)
+    X = rng.standard_normal((Cin, H, Wi, B)).astype(np.float32)
+    R = rng.standard_normal((Cout, H, Wi, B)).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    E = datagen.encode_dense(Wc)
+    g, og = hipabi.conv_geom(Cin, Cout, 3, 3, H, Wi, (1, 1), (1, 1)), ocg(Cin, Cout, 3, 3, H, Wi, (1, 1), (1, 1))
+    conv = oracle.conv2d_pf(as_oracle(E), og, X, B, b)
+    for act in ("none", "relu"):
+        want = oracle.act(oracle.add(conv, R), act)
+        assert np.array_equal(gpu_conv(ctx, E, g, X, B, b, act, window=window, residual=R), want)
+    want = oracle.act(oracle.add(conv, R), "tanh")
+    assert rel_err(gpu_conv(ctx, E, g, X, B, b, "tanh", window=window, residual=R), want) <= 1e-6
 
 
 def test_conv_reference_vectors(ctx, golden):

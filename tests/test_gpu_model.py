@@ -155,8 +155,10 @@ def test_cnn(backend, oracle, tmp_path, B):
     payload, t = cnn_model(rng, B)
     model = backend.SparseOnnxModel(ow.save(str(tmp_path / "cnn.onnx"), payload))
     desc = model.describe()
-    assert [d.split()[0] for d in desc] == ["Conv", "MaxPool", "Conv", "Conv", "Add", "GlobalAveragePool", "Gemm"]
-    assert "act=relu" in desc[0] and "act=relu" in desc[2] and "act=none" in desc[3] and "act=relu" in desc[6]
+    # the residual Add is fused into the second 3x3 convolution
+    assert [d.split()[0] for d in desc] == ["Conv", "MaxPool", "Conv", "Conv", "GlobalAveragePool", "Gemm"]
+    assert "act=relu" in desc[0] and "act=relu" in desc[2] and "act=none" in desc[3] and "+residual" in desc[3]
+    assert "act=relu" in desc[5]
     X = rng.standard_normal((B, 3, 16, 16)).astype(np.float32)
     Y = model.run(X)                                                         # C-order NCHW in, (B, 10) out
     assert Y.shape == (B, 10)
@@ -244,7 +246,9 @@ def test_resnet18_shaped(backend, oracle, tmp_path):
     payload, t = datagen.resnet18_onnx(seed=47, batch=4, hw=64, sparsity=0.8, classes=100, width=32)
     model = backend.SparseOnnxModel(ow.save(str(tmp_path / "r18.onnx"), payload))
     desc = model.describe()
-    assert sum(d.startswith("Conv") for d in desc) == 20 and sum(d.startswith("Add") for d in desc) == 8
+    # every residual Add (and the ReLU after it) is fused into the convolution before it
+    assert sum(d.startswith("Conv") for d in desc) == 20 and sum("+residual" in d for d in desc) == 8
+    assert not any(d.startswith("Add") or d.startswith("Relu") for d in desc)
     assert model.output_shape() == [4, 100]
     X = np.random.default_rng(1).standard_normal((4, 3, 64, 64)).astype(np.float32)
     Y = model.run(X)
