@@ -172,7 +172,8 @@ def test_conv_plan_validation(ctx):
 
 
 @pytest.mark.parametrize("C,H,Wi,B,k,s,p", [(3, 8, 8, 2, (2, 2), (2, 2), (0, 0)), (4, 9, 7, 3, (3, 3), (2, 2), (1, 1)),
-                                           (2, 5, 6, 1, (3, 2), (1, 1), (1, 0)), (64, 56, 56, 8, (3, 3), (2, 2), (1, 1))])
+                                           (2, 5, 6, 1, (3, 2), (1, 1), (1, 0)), (64, 56, 56, 8, (3, 3), (2, 2), (1, 1)),
+                                           (5, 11, 13, 4, (3, 3), (2, 2), (1, 1)), (3, 7, 7, 12, (2, 3), (1, 2), (0, 1))])
 def test_maxpool(ctx, oracle, C, H, Wi, B, k, s, p):
     rng = np.random.default_rng(C + H)
     X = rng.standard_normal((C, H, Wi, B)).astype(np.float32)
