@@ -223,7 +223,27 @@ def bench_mlp(steps, warmup, with_cpu=True):
             "nnz_gflops_device_resident": round(model.nnz_flops_per_sample() * 256 / (dev_ms * 1e-3) / 1e9, 1)}
 
 
-def bench_cnn(steps, warmup):
+def cpu_baseline_cnn(payload, model, sample=4):
+    """The same graph, layer by layer, with the plain-C restatement of the reference's conv /
+    pool / add / FC kernels on the host cores (the reference's own model runtime needs
+    libprotobuf and is not buildable here, hence kind "port"), on a bounded sample of the batch.
+    Also compares the GPU's output for those images with the CPU's, bit for bit."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    from graph_oracle import run_graph
+    from oracle import Oracle
+    orc = Oracle()
+    X = np.random.default_rng(5).standard_normal((32, 3, 224, 224)).astype(np.float32)
+    y_gpu = model.run(X)
+    t0 = time.perf_counter()
+    y_cpu = run_graph(orc, payload, X[:sample])
+    dt = time.perf_counter() - t0
+    return {"samples_per_s": round(sample / dt, 2), "ms_per_image": round(dt / sample * 1e3, 1), "kind": "port",
+            "cores": orc.num_threads(), "sample": "%d of the 32 images, one pass" % sample,
+            "gpu_bit_exact_vs_cpu": bool(np.array_equal(y_cpu, y_gpu[:sample])),
+            "gpu_max_rel_err_vs_cpu": float(np.abs(y_cpu.astype(np.float64) - y_gpu[:sample]).max() / max(np.abs(y_cpu).max(), 1e-30))}
+
+
+def bench_cnn(steps, warmup, with_cpu=True):
     import datagen
     import onnx_wire as ow
     import sparseops_backend as sb
@@ -233,6 +253,7 @@ def bench_cnn(steps, warmup):
     dev_ms = model.time_device(steps, warmup)
     flops = model.nnz_flops_per_sample() * 32
     return {"workload": "ResNet-18-shaped conv stack (no BN), 80% sparse, B=32, 3x224x224, implicit im2col",
+            "cpu_baseline": cpu_baseline_cnn(payload, model) if with_cpu else None,
             "layers": len(model.describe()), "ms_per_batch_device_resident": round(dev_ms, 3),
             "samples_per_s_device_resident": round(32 / (dev_ms * 1e-3), 1),
             "nnz_gflop_per_batch": round(flops / 1e9, 2), "nnz_gflops": round(flops / (dev_ms * 1e-3) / 1e9, 1)}
@@ -330,7 +351,7 @@ def main():
         log("sparse MLP ...")
         extras["mlp"] = bench_mlp(k, args.warmup, with_cpu=not args.no_cpu)
         log("sparse CNN ...")
-        extras["cnn"] = bench_cnn(max(5, args.steps // 20), 2)
+        extras["cnn"] = bench_cnn(max(5, args.steps // 20), 2, with_cpu=not args.no_cpu)
         result["extras"] = extras
     ctx.close()
     print(json.dumps(result), flush=True)
