@@ -153,6 +153,12 @@ typedef struct so_conv_plan so_conv_plan;
 so_status so_conv_plan_create(so_ctx *ctx, const so_ellpack *E, const so_conv_geom *g,
                               so_conv_plan **out);
 so_status so_conv_plan_free(so_ctx *ctx, so_conv_plan *plan);
+/* Re-sizes the plan's internal layouts for launches with batch B (how many output channels
+ * a wave takes depends on how many workgroups the batch yields).  Optional: results never
+ * depend on it; plans are created for batch 32.  Not to be called while a launch that uses
+ * the plan may be in flight on another stream, nor during graph capture (it allocates).
+ * No counterpart in the reference. */
+so_status so_conv_plan_tune(so_ctx *ctx, so_conv_plan *plan, uint32_t B);
 /* The LDS-windowed kernel's parameters for this plan (no counterpart in the reference:
  * a tuning/inspection aid): out = {tile_h, tile_w, window_h, window_w, channels per
  * chunk, chunks, output channels per wave, 0}; all zero when the geometry does not

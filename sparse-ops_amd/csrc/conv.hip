@@ -42,6 +42,7 @@ struct so_conv_window {
 };
 
 struct so_conv_plan {
+    uint32_t tuned_batch = 32;   // batch the windowed layout was sized for
     so_conv_geom g;
     const so_ellpack *E = nullptr;
     int2 *d_taps = nullptr;  // per slot: x = (cin*H + dh)*W + dw (elements of B floats), y = dh<<16 | (dw & 0xffff)
@@ -461,7 +462,7 @@ void conv_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_
 // hold enough nonzeros to amortise its copy and barrier; the whole output must give the chip
 // enough workgroups at batch tile 32).
 so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32_t> &idx,
-                       const std::vector<uint32_t> &nnz, const std::vector<float> &Wd)
+                       const std::vector<uint32_t> &nnz, const std::vector<float> &Wd, uint32_t batch)
 {
     const so_conv_geom &g = plan->g;
     const so_ellpack *E = plan->E;
@@ -511,7 +512,7 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     double best_cost = 0.0;
     for (int cpw : {8, 4, 2, 1}) {
         if (cpw > cpw_max && cpw != 1) continue;
-        const uint64_t wgs = window_workgroups(w, g.Cout, (uint32_t)cpw, 32);
+        const uint64_t wgs = window_workgroups(w, g.Cout, (uint32_t)cpw, batch);
         const double rounds = (double)so_ceil_div((uint32_t)std::min<uint64_t>(wgs, 1u << 30), (uint32_t)ctx->compute_units);
         const double cost = rounds * cpw * (6.5 + 10.0 / cpw + 29.0 / run);
         if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; w.cpw = cpw; }
@@ -635,7 +636,7 @@ extern "C" so_status so_conv_plan_create(so_ctx *ctx, const so_ellpack *E, const
         return s;
     }
     plan->d_taps = (int2 *)d;
-    s = build_window(ctx, plan, idx, nnz, Wd);
+    s = build_window(ctx, plan, idx, nnz, Wd, 32);
     if (s != SO_OK) {
         (void)hipFree(plan->d_taps);
         delete plan;
@@ -645,16 +646,40 @@ extern "C" so_status so_conv_plan_create(so_ctx *ctx, const so_ellpack *E, const
     return SO_OK;
 }
 
+static void free_window(so_conv_plan *plan)
+{
+    if (plan->win.d_stream) (void)hipFree(plan->win.d_stream);
+    if (plan->win.d_gbase) (void)hipFree(plan->win.d_gbase);
+    if (plan->win.d_quads) (void)hipFree(plan->win.d_quads);
+    plan->win = so_conv_window();
+}
+
 extern "C" so_status so_conv_plan_free(so_ctx *ctx, so_conv_plan *plan)
 {
     if (!plan) return SO_OK;
     if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (plan->d_taps) (void)hipFree(plan->d_taps);
-    if (plan->win.d_stream) (void)hipFree(plan->win.d_stream);
-    if (plan->win.d_gbase) (void)hipFree(plan->win.d_gbase);
-    if (plan->win.d_quads) (void)hipFree(plan->win.d_quads);
+    free_window(plan);
     delete plan;
     return SO_OK;
+}
+
+extern "C" so_status so_conv_plan_tune(so_ctx *ctx, so_conv_plan *plan, uint32_t B)
+{
+    SO_REQUIRE(ctx && plan, "so_conv_plan_tune: null argument");
+    // The layout depends on the batch only through the number of batch tiles of 16.
+    const uint32_t batch = std::max(kWinBT, B / kWinBT * kWinBT);
+    if (batch == plan->tuned_batch) return SO_OK;
+    const so_ellpack *E = plan->E;
+    const size_t slots = (size_t)E->m * E->r;
+    std::vector<uint32_t> idx(slots), nnz(E->m);
+    std::vector<float> Wd(slots);
+    so_status s = so_ellpack_download(ctx, E, SO_LAYOUT_ROW, Wd.data(), idx.data(), nnz.data());
+    if (s != SO_OK) return s;
+    SO_HIP(hipStreamSynchronize(ctx->stream));      // no launch may still be reading the old arrays
+    free_window(plan);
+    plan->tuned_batch = batch;
+    return build_window(ctx, plan, idx, nnz, Wd, batch);
 }
 
 extern "C" so_status so_conv_plan_window(const so_conv_plan *plan, uint32_t out[8])

@@ -19,7 +19,7 @@ LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS, LAYOUT_TILED = 1, 2, 4, 8
 SYMBOLS = (
     "so_device_count so_init so_destroy so_last_error so_device_info so_malloc so_free so_h2d so_d2h "
     "so_d2d so_fill_zero so_sync so_timer_begin so_timer_end so_ellpack_upload so_ellpack_free "
-    "so_ellpack_dims so_ellpack_download so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv2d_add "
+    "so_ellpack_dims so_ellpack_download so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
     "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_graph_begin so_graph_end "
     "so_graph_launch so_graph_free").split()
 
@@ -80,6 +80,7 @@ def load_library(path=None):
         "so_conv_plan_create": [_vp, _vp, ct.POINTER(ConvGeom), ct.POINTER(_vp)],
         "so_conv_plan_free": [_vp, _vp],
         "so_conv_plan_window": [_vp, ct.POINTER(ct.c_uint32)],
+        "so_conv_plan_tune": [_vp, _vp, ct.c_uint32],
         "so_conv2d": [_vp, _vp, _vp, _u32, _vp, _vp, ct.c_int],
         "so_conv2d_add": [_vp, _vp, _vp, ct.c_uint32, _vp, _vp, _vp, ct.c_int],
         "so_maxpool": [_vp, ct.POINTER(PoolGeom), _vp, _u32, _vp],
@@ -209,6 +210,9 @@ class Context:
         h = _vp()
         self._ck(self.lib.so_conv_plan_create(self.h, E.h, ct.byref(geom), ct.byref(h)))
         return h.value
+
+    def conv_plan_tune(self, plan, B):
+        self._ck(self.lib.so_conv_plan_tune(self.h, plan, B))
 
     def conv_plan_window(self, plan):
         """-> dict of the LDS-windowed kernel's parameters, or None when the plan has none."""

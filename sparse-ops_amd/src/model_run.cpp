@@ -28,6 +28,8 @@ void SparseOnnxModel::resize_buffers(uint32_t batch)
     M.stage_in.reserve(M.in_features * batch * sizeof(float));
     M.stage_out.reserve(M.out_features * batch * sizeof(float));
     M.batch = batch;
+    for (const LayerPlan &L : M.layers)
+        if (L.conv) check(so_conv_plan_tune(ctx, L.conv, batch), "so_conv_plan_tune");
     if (M.use_graph && !M.layers.empty()) {
         check(so_graph_begin(ctx), "so_graph_begin");
         try {

@@ -123,6 +123,32 @@ def test_conv_with_fused_residual_add(ctx, oracle, B, window):
     assert rel_err(gpu_conv(ctx, E, g, X, B, b, "tanh", window=window, residual=R), want) <= 1e-6
 
 
+def test_conv_plan_tune_changes_layout_not_results(ctx, oracle):
+    """so_conv_plan_tune re-sizes the windowed layout for a batch; outputs keep their bits."""
+    from oracle import conv_geom as ocg
+    rng = np.random.default_rng(77)
+    Cin, Cout, H, Wi = 32, 64, 56, 56
+    Wc = sparse_matrix(rng, Cout, Cin * 9, .8)
+    E = datagen.encode_dense(Wc)
+    g, og = hipabi.conv_geom(Cin, Cout, 3, 3, H, Wi, (1, 1), (1, 1)), ocg(Cin, Cout, 3, 3, H, Wi, (1, 1), (1, 1))
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+    plan = ctx.conv_plan(dE, g)
+    seen = set()
+    for B in (16, 32, 128, 16):
+        ctx.conv_plan_tune(plan, B)
+        seen.add(ctx.conv_plan_window(plan)["channels_per_wave"])
+        Bx = 16                                           # results for a batch of 16 under every tuning
+        X = rng.standard_normal((Cin, H, Wi, Bx)).astype(np.float32)
+        dX, dY = ctx.array(X), ctx.empty((Cout, H, Wi, Bx))
+        ctx.conv2d(plan, dX, Bx, None, dY, "relu")
+        assert np.array_equal(dY.download(), oracle.conv2d_pf(as_oracle(E), og, X, Bx, None, "relu"))
+        dX.free()
+        dY.free()
+    assert len(seen) > 1                                  # fewer channels per wave for the small batch
+    ctx.conv_plan_free(plan)
+    dE.free()
+
+
 def test_conv_reference_vectors(ctx, golden):
     for i, c in enumerate(golden["conv_cases"]):
         Cin, Cout, H, Wi, B = (int(v) for v in c[:5])
