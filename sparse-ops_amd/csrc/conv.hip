@@ -198,8 +198,11 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
 // chunk t is computed.
 constexpr int kWinThreads = 1024;
 constexpr int kWinMaxPerThread = 6;   // float4 window elements a thread copies per chunk
-constexpr uint32_t kWinLPP = 4;       // lanes per pixel
-constexpr uint32_t kWinBT = 4 * kWinLPP;   // batch tile
+constexpr uint32_t kWinLPP = 4;       // lanes per pixel of the preferred batch tile ...
+constexpr uint32_t kWinBT = 4 * kWinLPP;   // ... of 16; batches that are only multiples of 8 or 4 use tiles of 8 or 4
+
+// Lanes per pixel for batch B: the largest batch tile (16, 8, 4) that divides B; 0 if none does.
+inline uint32_t window_lpp(uint32_t B) { return B % 16 == 0 ? 4u : B % 8 == 0 ? 2u : B % 4 == 0 ? 1u : 0u; }
 
 struct WinArgs {
     uint32_t TH, TW, IH, IW, cc, nch, tiles_x, pg, cg, groups;
@@ -392,10 +395,12 @@ so_status window_configure(so_ctx *ctx)
 {
     static bool configured = false;
     if (configured) return SO_OK;
-    SO_HIP((window_allow_lds<8, kWinLPP>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<4, kWinLPP>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<2, kWinLPP>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<1, kWinLPP>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<8, 4>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<4, 4>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<2, 4>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<1, 4>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<8, 2>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<4, 2>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<2, 2>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<1, 2>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<8, 1>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<4, 1>(ctx->max_lds_bytes)));
+    SO_HIP((window_allow_lds<2, 1>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<1, 1>(ctx->max_lds_bytes)));
     configured = true;
     return SO_OK;
 }
@@ -403,35 +408,37 @@ so_status window_configure(so_ctx *ctx)
 // Workgroups the windowed kernel launches for batch B with `cpw` channels per wave.
 uint64_t window_workgroups(const so_conv_window &w, uint32_t cout, uint32_t cpw, uint32_t B)
 {
-    const uint32_t pg = so_ceil_div(w.TH * w.TW, 64u / kWinLPP), cg = 16u / pg;
-    return (uint64_t)w.tiles_x * w.tiles_y * so_ceil_div(so_ceil_div(cout, cpw), cg) * (B / kWinBT);
+    const uint32_t lpp = std::max(1u, window_lpp(B));
+    const uint32_t pg = so_ceil_div(w.TH * w.TW, 64u / lpp), cg = 16u / pg;
+    return (uint64_t)w.tiles_x * w.tiles_y * so_ceil_div(so_ceil_div(cout, cpw), cg) * std::max(1u, B / (4u * lpp));
 }
 
 // Launches the windowed kernel if the plan has the layout, the batch suits it and the grid
 // covers the chip; *done says whether it did.
+template <uint32_t LPP>
 so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B, const float *dBias,
                         const float *dResid, float *dY, int act, bool forced, bool *done)
 {
     const so_conv_window &w = plan->win;
-    constexpr uint32_t PPW = 64 / kWinLPP;
+    constexpr uint32_t PPW = 64 / LPP;
     WinArgs a;
     a.TH = w.TH; a.TW = w.TW; a.IH = w.IH; a.IW = w.IW; a.cc = w.cc; a.nch = w.nch; a.tiles_x = w.tiles_x;
     a.groups = w.groups;
     a.pg = so_ceil_div(w.TH * w.TW, PPW);
     a.cg = 16 / a.pg;
-    a.win_f4 = w.cc * w.IH * w.IW * kWinLPP;
-    a.buf_f4 = (w.cc + 1) * w.IH * w.IW * kWinLPP;
+    a.win_f4 = w.cc * w.IH * w.IW * LPP;
+    a.buf_f4 = (w.cc + 1) * w.IH * w.IW * LPP;
     a.nbuf = w.nch > 1 ? 2u : 1u;
     const size_t lds = (size_t)a.nbuf * a.buf_f4 * 16;
-    const dim3 grid(w.tiles_x * w.tiles_y, so_ceil_div(w.groups, a.cg), B / kWinBT);
+    const dim3 grid(w.tiles_x * w.tiles_y, so_ceil_div(w.groups, a.cg), B / (4 * LPP));
     const uint64_t wgs = (uint64_t)grid.x * grid.y * grid.z;
     if (!forced && 2 * wgs < (uint64_t)ctx->compute_units) return SO_OK;      // too few workgroups for the chip
     if (grid.y > 65535u || grid.z > 65535u) return SO_OK;
     switch (w.cpw) {
-    case 8:  window_launch_act<8, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
-    case 4:  window_launch_act<4, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
-    case 2:  window_launch_act<2, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
-    default: window_launch_act<1, kWinLPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
+    case 8:  window_launch_act<8, (int)LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
+    case 4:  window_launch_act<4, (int)LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
+    case 2:  window_launch_act<2, (int)LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
+    default: window_launch_act<1, (int)LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
     }
     *done = true;
     return SO_OK;
@@ -667,8 +674,8 @@ extern "C" so_status so_conv_plan_free(so_ctx *ctx, so_conv_plan *plan)
 extern "C" so_status so_conv_plan_tune(so_ctx *ctx, so_conv_plan *plan, uint32_t B)
 {
     SO_REQUIRE(ctx && plan, "so_conv_plan_tune: null argument");
-    // The layout depends on the batch only through the number of batch tiles of 16.
-    const uint32_t batch = std::max(kWinBT, B / kWinBT * kWinBT);
+    // The layout depends on the batch only through the number of batch tiles.
+    const uint32_t batch = std::max(4u, B / 4u * 4u);
     if (batch == plan->tuned_batch) return SO_OK;
     const so_ellpack *E = plan->E;
     const size_t slots = (size_t)E->m * E->r;
@@ -705,14 +712,17 @@ static so_status conv2d_dispatch(so_ctx *ctx, const so_conv_plan *plan, const fl
     const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY | (uintptr_t)dResid;
     int maxvec = 4;
     if (const char *e = getenv("SPARSEOPS_CONV_VEC")) maxvec = atoi(e);
-    // The LDS-windowed kernel when the plan carries its layout and the batch splits into tiles of 16
-    // (SPARSEOPS_CONV_WINDOW=1 forces it whenever possible, =0 forbids it: tuning and tests).
-    if (plan->win.cc != 0 && B % kWinBT == 0 && (align & 15) == 0 && (uint64_t)plan->win.cc * g.H_in * g.W_in * B < (1ull << 31)) {
+    // The LDS-windowed kernel when the plan carries its layout and the batch splits into tiles of
+    // 16, 8 or 4 (SPARSEOPS_CONV_WINDOW=1 forces it whenever possible, =0 forbids it: tuning and tests).
+    const uint32_t lpp = window_lpp(B);
+    if (plan->win.cc != 0 && lpp != 0 && (align & 15) == 0 && (uint64_t)plan->win.cc * g.H_in * g.W_in * B < (1ull << 31)) {
         const char *force = getenv("SPARSEOPS_CONV_WINDOW");
         const bool forced = force && force[0] == '1';
         if (!(force && force[0] == '0')) {
             bool done = false;
-            const so_status s = window_launch(ctx, plan, dX, B, dBias, dResid, dY, act, forced, &done);
+            const so_status s = lpp == 4 ? window_launch<4>(ctx, plan, dX, B, dBias, dResid, dY, act, forced, &done)
+                              : lpp == 2 ? window_launch<2>(ctx, plan, dX, B, dBias, dResid, dY, act, forced, &done)
+                                         : window_launch<1>(ctx, plan, dX, B, dBias, dResid, dY, act, forced, &done);
             if (s != SO_OK) return s;
             if (done) {
                 SO_LAUNCH_CHECK();

@@ -23,7 +23,7 @@ def gpu_conv(ctx, E, g, X, B, bias, act="none", window=None, residual=None):
     if window is not None:
         os.environ["SPARSEOPS_CONV_WINDOW"] = "1" if window else "0"
         if window:
-            assert ctx.conv_plan_window(plan) is not None and B % 16 == 0
+            assert ctx.conv_plan_window(plan) is not None and B % 4 == 0
     try:
         return _gpu_conv(ctx, dE, plan, g, X, B, bias, act, residual)
     finally:
@@ -78,6 +78,10 @@ WINDOW_CASES = [
     (2, 9, 9, 9, 32, (5, 5), (1, 1), (2, 2), (1, 1), .5),         # 5x5
     (64, 64, 8, 8, 16, (3, 3), (1, 1), (1, 1), (1, 1), .8),       # 10 chunks, image smaller than... one tile row
     (20, 6, 6, 6, 32, (1, 1), (1, 1), (0, 0), (1, 1), .3),        # 1x1 with enough nonzeros per chunk
+    (16, 32, 28, 28, 8, (3, 3), (1, 1), (1, 1), (1, 1), .7),      # batch tile 8
+    (9, 21, 13, 11, 24, (3, 3), (2, 2), (1, 1), (1, 1), .5),      # batch 24 = 3 tiles of 8
+    (16, 24, 30, 30, 4, (3, 3), (1, 1), (1, 1), (1, 1), .6),      # batch tile 4 (half the lanes of a wave idle)
+    (3, 64, 32, 32, 12, (7, 7), (2, 2), (3, 3), (1, 1), .7),      # batch 12 = 3 tiles of 4
 ]
 
 
@@ -102,7 +106,7 @@ def test_conv_lds_window_kernel(ctx, oracle, Cin, Cout, H, Wi, B, k, s, p, d, sp
     assert rel_err(gpu_conv(ctx, E, g, X, B, b, "tanh", window=True), oracle.conv2d_pf(as_oracle(E), og, X, B, b, "tanh")) <= 1e-6
 
 
-@pytest.mark.parametrize("B,window", [(3, False), (4, False), (32, False), (32, True), (16, True)])
+@pytest.mark.parametrize("B,window", [(3, False), (4, False), (32, False), (32, True), (16, True), (8, True), (4, True)])
 def test_conv_with_fused_residual_add(ctx, oracle, B, window):
     """so_conv2d_add == conv, then the reference's Add, then the activation: same bits as
     the three layers one after the other, in both convolution kernels."""
