@@ -70,10 +70,12 @@ __device__ __forceinline__ void conv_load(const float *p, float (&v)[VEC])
 
 // VEC consecutive columns per lane; B % VEC == 0, so a lane's columns belong to
 // one output pixel (same taps, same bounds test) and are VEC consecutive batch
-// entries: one 4*VEC-byte load per tap.  One batch of 8 taps in flight per wave:
-// a second batch in registers was measured slower (the 8 waves of a workgroup
-// share the input window through L1 and deeper queues evict it).
-template <int VEC, int ACT>
+// entries: one 4*VEC-byte load per tap.  One batch of U taps in flight per wave.
+// U = 8 when the chip is full of waves: a second batch in registers was measured
+// slower (the 8 waves of a workgroup share the input window through L1 and deeper
+// queues evict it).  U = 32 for launches of few waves (small batches, small
+// images), where a wave's own memory-level parallelism is all the latency hiding there is.
+template <int VEC, int ACT, int U>
 __global__ __launch_bounds__(kChannelsPerGroup * 64)
 void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict__ taps,
                             const uint32_t *__restrict__ nnz, uint32_t r, so_conv_geom g,
@@ -104,18 +106,66 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
         for (int v = 0; v < VEC; ++v) acc[v] = b0;
     }
 
-    if (__all(interior)) {
+    if constexpr (U == 32) {
+        // Few waves on the chip: latency is everything.  Two register batches of 16 taps, the next
+        // one issued before the current one is consumed, so tap fetch, address arithmetic, gathers
+        // and multiply-adds of neighbouring batches overlap.  Branch-free taps as in the border path.
+        constexpr int H = 16;
+        const float *__restrict__ xsafe = X + b;
+        float wa[H], wb[H], xa[H][VEC], xb[H][VEC];
+        bool oka[H], okb[H];
+        auto issue = [&](uint32_t j0, float (&w)[H], float (&x)[H][VEC], bool (&ok)[H]) {
+            int2 t[H];
+#pragma unroll
+            for (int u = 0; u < H; ++u) {       // all the scalar tap loads first, as one cluster
+                t[u] = trow[j0 + u];
+                w[u] = wrow[j0 + u];
+            }
+#pragma unroll
+            for (int u = 0; u < H; ++u) {
+                const int32_t hin = h0 + (t[u].y >> 16), win = w0 + (int32_t)(int16_t)(t[u].y & 0xffff);
+                ok[u] = (uint32_t)hin < g.H_in && (uint32_t)win < g.W_in;
+                conv_load<VEC>(ok[u] ? X + lanebase + (int64_t)t[u].x * (int64_t)B : xsafe, x[u]);
+            }
+        };
+        auto consume = [&](const float (&w)[H], const float (&x)[H][VEC], const bool (&ok)[H]) {
+#pragma unroll
+            for (int u = 0; u < H; ++u)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(w[u], ok[u] ? x[u][v] : 0.0f, acc[v]);
+        };
+        const uint32_t nb = cnt / H;
+        if (nb) issue(0, wa, xa, oka);
+        uint32_t bi = 0;
+        for (; bi + 1 < nb; bi += 2) {
+            issue((bi + 1) * H, wb, xb, okb);
+            consume(wa, xa, oka);
+            if (bi + 2 < nb) issue((bi + 2) * H, wa, xa, oka);
+            consume(wb, xb, okb);
+        }
+        if (nb & 1u) consume(wa, xa, oka);
+        for (uint32_t j = nb * H; j < cnt; ++j) {
+            const int2 t = trow[j];
+            const int32_t hin = h0 + (t.y >> 16), win = w0 + (int32_t)(int16_t)(t.y & 0xffff);
+            if ((uint32_t)hin < g.H_in && (uint32_t)win < g.W_in) {
+                float x[VEC];
+                conv_load<VEC>(X + lanebase + (int64_t)t.x * (int64_t)B, x);
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(wrow[j], x[v], acc[v]);
+            }
+        }
+    } else if (__all(interior)) {
         const float *__restrict__ xl = X + lanebase;
         uint32_t j = 0;
-        for (; j + 8 <= cnt; j += 8) {
-            float w[8], x[8][VEC];
+        for (; j + U <= cnt; j += U) {
+            float w[U], x[U][VEC];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < U; ++u) {
                 w[u] = wrow[j + u];
                 conv_load<VEC>(xl + (int64_t)trow[j + u].x * (int64_t)B, x[u]);
             }
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
+            for (int u = 0; u < U; ++u)
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(w[u], x[u][v], acc[v]);
         }
@@ -132,19 +182,23 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
         // fma(w, 0, acc) = acc, which is what skipping it gives.
         const float *__restrict__ xsafe = X + b;
         uint32_t j = 0;
-        for (; j + 8 <= cnt; j += 8) {
-            float w[8], x[8][VEC];
-            bool ok[8];
+        for (; j + U <= cnt; j += U) {
+            float w[U], x[U][VEC];
+            bool ok[U];
+            int2 t[U];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int2 t = trow[j + u];
+            for (int u = 0; u < U; ++u) {       // all the scalar tap loads first, as one cluster
+                t[u] = trow[j + u];
                 w[u] = wrow[j + u];
-                const int32_t hin = h0 + (t.y >> 16), win = w0 + (int32_t)(int16_t)(t.y & 0xffff);
-                ok[u] = (uint32_t)hin < g.H_in && (uint32_t)win < g.W_in;
-                conv_load<VEC>(ok[u] ? X + lanebase + (int64_t)t.x * (int64_t)B : xsafe, x[u]);
             }
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
+            for (int u = 0; u < U; ++u) {
+                const int32_t hin = h0 + (t[u].y >> 16), win = w0 + (int32_t)(int16_t)(t[u].y & 0xffff);
+                ok[u] = (uint32_t)hin < g.H_in && (uint32_t)win < g.W_in;
+                conv_load<VEC>(ok[u] ? X + lanebase + (int64_t)t[u].x * (int64_t)B : xsafe, x[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(w[u], ok[u] ? x[u][v] : 0.0f, acc[v]);
         }
@@ -451,9 +505,17 @@ void conv_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_
     const so_conv_geom &g = plan->g;
     const so_ellpack *E = plan->E;
     const dim3 grid((uint32_t)((ncols + 64ull * VEC - 1) / (64ull * VEC)), so_ceil_div(g.Cout, kChannelsPerGroup));
+    // at most 4 waves per SIMD in the whole launch and rows long enough for a batch of 32
+    const bool few = (uint64_t)grid.x * g.Cout <= 16ull * (uint64_t)ctx->compute_units && E->max_nnz >= 64;
 #define SO_CONV_LAUNCH(A)                                                                          \
-    conv2d_implicit_kernel<VEC, A><<<grid, kChannelsPerGroup * 64, 0, ctx->stream>>>(              \
-        E->d_Wd, plan->d_taps, E->d_nnz, E->r, g, dX, B, ncols, dBias, dResid, dY)
+    do {                                                                                           \
+        if (few)                                                                                   \
+            conv2d_implicit_kernel<VEC, A, 32><<<grid, kChannelsPerGroup * 64, 0, ctx->stream>>>(  \
+                E->d_Wd, plan->d_taps, E->d_nnz, E->r, g, dX, B, ncols, dBias, dResid, dY);        \
+        else                                                                                       \
+            conv2d_implicit_kernel<VEC, A, 8><<<grid, kChannelsPerGroup * 64, 0, ctx->stream>>>(   \
+                E->d_Wd, plan->d_taps, E->d_nnz, E->r, g, dX, B, ncols, dBias, dResid, dY);        \
+    } while (0)
     switch (act) {
     case SO_ACT_RELU:    SO_CONV_LAUNCH(SO_ACT_RELU); break;
     case SO_ACT_SIGMOID: SO_CONV_LAUNCH(SO_ACT_SIGMOID); break;
