@@ -111,7 +111,6 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
         // one issued before the current one is consumed, so tap fetch, address arithmetic, gathers
         // and multiply-adds of neighbouring batches overlap.  Branch-free taps as in the border path.
         constexpr int H = 16;
-        const float *__restrict__ xsafe = X + b;
         float wa[H], wb[H], xa[H][VEC], xb[H][VEC];
         bool oka[H], okb[H];
         auto issue = [&](uint32_t j0, float (&w)[H], float (&x)[H][VEC], bool (&ok)[H]) {
@@ -124,8 +123,9 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
 #pragma unroll
             for (int u = 0; u < H; ++u) {
                 const int32_t hin = h0 + (t[u].y >> 16), win = w0 + (int32_t)(int16_t)(t[u].y & 0xffff);
-                ok[u] = (uint32_t)hin < g.H_in && (uint32_t)win < g.W_in;
-                conv_load<VEC>(ok[u] ? X + lanebase + (int64_t)t[u].x * (int64_t)B : xsafe, x[u]);
+                ok[u] = ((uint32_t)hin < g.H_in) & ((uint32_t)win < g.W_in);      // '&': no branch per tap
+                const int64_t off = lanebase + (int64_t)t[u].x * (int64_t)B;
+                conv_load<VEC>(X + (ok[u] ? off : (int64_t)b), x[u]);
             }
         };
         auto consume = [&](const float (&w)[H], const float (&x)[H][VEC], const bool (&ok)[H]) {
@@ -180,7 +180,6 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
         // branches: a tap that is out of bounds for a lane loads a harmless in-bounds
         // address (the lane's own batch entry of pixel (0,0,0)) and contributes
         // fma(w, 0, acc) = acc, which is what skipping it gives.
-        const float *__restrict__ xsafe = X + b;
         uint32_t j = 0;
         for (; j + U <= cnt; j += U) {
             float w[U], x[U][VEC];
@@ -194,8 +193,9 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int32_t hin = h0 + (t[u].y >> 16), win = w0 + (int32_t)(int16_t)(t[u].y & 0xffff);
-                ok[u] = (uint32_t)hin < g.H_in && (uint32_t)win < g.W_in;
-                conv_load<VEC>(ok[u] ? X + lanebase + (int64_t)t[u].x * (int64_t)B : xsafe, x[u]);
+                ok[u] = ((uint32_t)hin < g.H_in) & ((uint32_t)win < g.W_in);      // '&': no branch per tap
+                const int64_t off = lanebase + (int64_t)t[u].x * (int64_t)B;
+                conv_load<VEC>(X + (ok[u] ? off : (int64_t)b), x[u]);
             }
 #pragma unroll
             for (int u = 0; u < U; ++u)
