@@ -281,3 +281,20 @@ def test_torch_exported_models(backend, oracle, name):
     # a second batch through the same model object, in Fortran order
     Y2 = model.run(np.asfortranarray(X[::-1].copy()))
     assert rel_err(Y2, Yt[::-1]) <= 1e-5
+
+
+def test_resnet18_full_size_batch_independence(backend, oracle, tmp_path):
+    """Config 5 at its real size (ResNet-18-shaped, 224x224, 80 % sparse): every image's output is
+    independent of the batch it travels in.  Batches of 32, 16, 8 and 3 take differently tuned
+    convolution kernels (channels per wave, batch tile, gather kernel), and all must give the same
+    bits; the oracle pins those bits for the first image."""
+    payload, _ = datagen.resnet18_onnx(seed=47, batch=32, hw=224, sparsity=0.8)
+    model = backend.SparseOnnxModel(ow.save(str(tmp_path / "r18.onnx"), payload))
+    X = np.random.default_rng(3).standard_normal((32, 3, 224, 224)).astype(np.float32)
+    Y = model.run(X)
+    assert Y.shape == (32, 1000) and np.isfinite(Y).all()
+    for B in (16, 8, 3):
+        assert np.array_equal(model.run(X[:B]), Y[:B]), B
+    assert np.array_equal(model.run(X), Y)                       # back to 32 after the resizes
+    from graph_oracle import run_graph
+    assert np.array_equal(run_graph(oracle, payload, X[:1]), Y[:1])
