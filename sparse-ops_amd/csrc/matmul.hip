@@ -129,12 +129,34 @@ void ellpack_matmul_kernel(const float *__restrict__ Wd, const uint32_t *__restr
         consume(wb, xb);
     }
     if (nb & 1u) consume(wa, xa);
-    for (uint32_t j = nb * kUnroll; j < cnt; ++j) {
-        const float w = wrow[j];
-        float x[VEC];
-        load_vec<VEC>(xcol + (size_t)irow[j] * C, x);
+    // The last, partial batch.  With few waves on the chip (kUnroll 32) all its gathers are issued at
+    // once (slots past the row's end re-read the row's last nonzero) and the multiply-adds run under
+    // a wave-uniform test per slot: one memory round trip instead of one per nonzero.  With the chip
+    // full of waves the plain loop is faster (no redundant gathers; other waves hide the latency).
+    if constexpr (kUnroll >= 32) {
+        if (const uint32_t rem = cnt - nb * kUnroll) {
+            const uint32_t j0 = nb * kUnroll;
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(w, x[v], acc[v]);
+            for (int u = 0; u < kUnroll; ++u) {
+                const uint32_t j = j0 + min((uint32_t)u, rem - 1u);
+                wa[u] = wrow[j];
+                load_vec<VEC>(xcol + (size_t)irow[j] * C, xa[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+                if ((uint32_t)u < rem) {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(wa[u], xa[u][v], acc[v]);
+                }
+        }
+    } else {
+        for (uint32_t j = nb * kUnroll; j < cnt; ++j) {
+            const float w = wrow[j];
+            float x[VEC];
+            load_vec<VEC>(xcol + (size_t)irow[j] * C, x);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(w, x[v], acc[v]);
+        }
     }
 
     if (live) {
