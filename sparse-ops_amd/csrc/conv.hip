@@ -144,15 +144,30 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
             consume(wb, xb, okb);
         }
         if (nb & 1u) consume(wa, xa, oka);
-        for (uint32_t j = nb * H; j < cnt; ++j) {
-            const int2 t = trow[j];
-            const int32_t hin = h0 + (t.y >> 16), win = w0 + (int32_t)(int16_t)(t.y & 0xffff);
-            if ((uint32_t)hin < g.H_in && (uint32_t)win < g.W_in) {
-                float x[VEC];
-                conv_load<VEC>(X + lanebase + (int64_t)t.x * (int64_t)B, x);
+        // the partial last batch in one round trip: slots past the end re-read the last tap and are
+        // dropped by a wave-uniform test
+        if (const uint32_t rem = cnt - nb * H) {
+            const uint32_t j0 = nb * H;
+            int2 t[H];
 #pragma unroll
-                for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(wrow[j], x[v], acc[v]);
+            for (int u = 0; u < H; ++u) {
+                const uint32_t j = j0 + min((uint32_t)u, rem - 1u);
+                t[u] = trow[j];
+                wa[u] = wrow[j];
             }
+#pragma unroll
+            for (int u = 0; u < H; ++u) {
+                const int32_t hin = h0 + (t[u].y >> 16), win = w0 + (int32_t)(int16_t)(t[u].y & 0xffff);
+                oka[u] = ((uint32_t)hin < g.H_in) & ((uint32_t)win < g.W_in);
+                const int64_t off = lanebase + (int64_t)t[u].x * (int64_t)B;
+                conv_load<VEC>(X + (oka[u] ? off : (int64_t)b), xa[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < H; ++u)
+                if ((uint32_t)u < rem) {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(wa[u], oka[u] ? xa[u][v] : 0.0f, acc[v]);
+                }
         }
     } else if (__all(interior)) {
         const float *__restrict__ xl = X + lanebase;
