@@ -195,22 +195,18 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
         // branches: a tap that is out of bounds for a lane loads a harmless in-bounds
         // address (the lane's own batch entry of pixel (0,0,0)) and contributes
         // fma(w, 0, acc) = acc, which is what skipping it gives.
+        const float *__restrict__ xsafe = X + b;
         uint32_t j = 0;
         for (; j + U <= cnt; j += U) {
             float w[U], x[U][VEC];
             bool ok[U];
-            int2 t[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {       // all the scalar tap loads first, as one cluster
-                t[u] = trow[j + u];
-                w[u] = wrow[j + u];
-            }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int32_t hin = h0 + (t[u].y >> 16), win = w0 + (int32_t)(int16_t)(t[u].y & 0xffff);
-                ok[u] = ((uint32_t)hin < g.H_in) & ((uint32_t)win < g.W_in);      // '&': no branch per tap
-                const int64_t off = lanebase + (int64_t)t[u].x * (int64_t)B;
-                conv_load<VEC>(X + (ok[u] ? off : (int64_t)b), x[u]);
+                const int2 t = trow[j + u];
+                w[u] = wrow[j + u];
+                const int32_t hin = h0 + (t.y >> 16), win = w0 + (int32_t)(int16_t)(t.y & 0xffff);
+                ok[u] = (uint32_t)hin < g.H_in && (uint32_t)win < g.W_in;
+                conv_load<VEC>(ok[u] ? X + lanebase + (int64_t)t.x * (int64_t)B : xsafe, x[u]);
             }
 #pragma unroll
             for (int u = 0; u < U; ++u)
@@ -522,8 +518,8 @@ void conv_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_
     const so_conv_geom &g = plan->g;
     const so_ellpack *E = plan->E;
     const dim3 grid((uint32_t)((ncols + 64ull * VEC - 1) / (64ull * VEC)), so_ceil_div(g.Cout, kChannelsPerGroup));
-    // at most 4 waves per SIMD in the whole launch and rows long enough for a batch of 32
-    const bool few = (uint64_t)grid.x * g.Cout <= 16ull * (uint64_t)ctx->compute_units && E->max_nnz >= 64;
+    // at most 2 waves per SIMD in the whole launch and rows long enough for its batches
+    const bool few = (uint64_t)grid.x * g.Cout <= 8ull * (uint64_t)ctx->compute_units && E->max_nnz >= 64;
 #define SO_CONV_LAUNCH(A)                                                                          \
     do {                                                                                           \
         if (few)                                                                                   \
