@@ -84,7 +84,15 @@ void gap_kernel(uint32_t C, uint32_t HW, const float *__restrict__ X, uint32_t B
         const uint64_t c = q / B;
         const float *xp = X + c * HW * B + b;
         float s = 0.0f;
-        for (uint32_t i = 0; i < HW; ++i) s = s + xp[(uint64_t)i * B];
+        uint32_t i = 0;
+        for (; i + 8 <= HW; i += 8) {            // eight loads in flight, the additions still in order
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = xp[(uint64_t)(i + u) * B];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s = s + v[u];
+        }
+        for (; i < HW; ++i) s = s + xp[(uint64_t)i * B];
         Y[q] = s * scale;
     }
 }
