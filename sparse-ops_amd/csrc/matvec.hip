@@ -49,10 +49,50 @@ __device__ __forceinline__ const float *stage_x(const float *__restrict__ x, uin
     return lds;
 }
 
-// Dot product of one row with x, computed by a whole wave.  The row's slots
-// [beg, end) are covered by aligned groups of four; a lane loads up to four such
-// groups before using any (addresses past the row are clamped onto its last
-// group and every slot outside [beg, end) is masked to an exact no-op).
+// Dot product of one row with x, computed by a whole wave, in two halves so that a caller can
+// put other work (staging x, finishing the previous row) between issuing the loads and using
+// them.  The row's slots [beg, end) are covered by aligned groups of four; a lane loads up to four
+// such groups (addresses past the row are clamped onto its last group and every slot outside
+// [beg, end) is masked to an exact no-op).  Rows longer than 1024 slots continue in row_rest.
+struct RowLoads {
+    f32x4 w[4];
+    u32x4 c[4];
+};
+
+__device__ __forceinline__ void row_issue(const f32x4 *__restrict__ Wd4, const u32x4 *__restrict__ idx4,
+                                          uint64_t beg, uint64_t end, uint64_t q0, RowLoads &L)
+{
+    const uint64_t qlast = end > beg ? (end - 1) >> 2 : beg >> 2;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const uint64_t q = std::min<uint64_t>(q0 + 64u * u, qlast);
+        L.w[u] = __builtin_nontemporal_load(Wd4 + q);
+        L.c[u] = __builtin_nontemporal_load(idx4 + q);
+    }
+}
+
+__device__ __forceinline__ void row_consume(const RowLoads &L, uint64_t beg, uint64_t end, uint64_t q0, const float *xs,
+                                            float &a0, float &a1, float &a2, float &a3)
+{
+    // slot k of group u is live iff its distance from the row's start is in [0, end - beg): one
+    // unsigned 32-bit comparison (a slot before the row gives a huge distance)
+    const uint32_t len = (uint32_t)(end - beg);
+    const int32_t rel0 = (int32_t)(int64_t)((q0 << 2) - beg);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const int32_t rel = rel0 + 256 * u;
+        const bool v0 = (uint32_t)rel < len, v1 = (uint32_t)(rel + 1) < len;
+        const bool v2 = (uint32_t)(rel + 2) < len, v3 = (uint32_t)(rel + 3) < len;
+        const float x0 = xs[v0 ? L.c[u].x : 0u], x1 = xs[v1 ? L.c[u].y : 0u];
+        const float x2 = xs[v2 ? L.c[u].z : 0u], x3 = xs[v3 ? L.c[u].w : 0u];
+        a0 = __builtin_fmaf(v0 ? L.w[u].x : 0.0f, v0 ? x0 : 0.0f, a0);
+        a1 = __builtin_fmaf(v1 ? L.w[u].y : 0.0f, v1 ? x1 : 0.0f, a1);
+        a2 = __builtin_fmaf(v2 ? L.w[u].z : 0.0f, v2 ? x2 : 0.0f, a2);
+        a3 = __builtin_fmaf(v3 ? L.w[u].w : 0.0f, v3 ? x3 : 0.0f, a3);
+    }
+}
+
+// The whole row at once (used where rows are not pipelined).
 __device__ __forceinline__ float wave_row_dot(const f32x4 *__restrict__ Wd4, const u32x4 *__restrict__ idx4,
                                               uint64_t beg, uint64_t end, const float *xs, uint32_t lane)
 {
@@ -60,26 +100,9 @@ __device__ __forceinline__ float wave_row_dot(const f32x4 *__restrict__ Wd4, con
     if (end == beg) return 0.0f;
     const uint64_t qlast = (end - 1) >> 2;
     for (uint64_t q0 = (beg >> 2) + lane; q0 <= qlast; q0 += 256) {
-        f32x4 w[4];
-        u32x4 c[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const uint64_t q = std::min<uint64_t>(q0 + 64u * u, qlast);
-            w[u] = __builtin_nontemporal_load(Wd4 + q);
-            c[u] = __builtin_nontemporal_load(idx4 + q);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const uint64_t e = (q0 + 64u * u) << 2;
-            const bool v0 = e >= beg && e < end, v1 = e + 1 >= beg && e + 1 < end;
-            const bool v2 = e + 2 >= beg && e + 2 < end, v3 = e + 3 >= beg && e + 3 < end;
-            const float x0 = xs[v0 ? c[u].x : 0u], x1 = xs[v1 ? c[u].y : 0u];
-            const float x2 = xs[v2 ? c[u].z : 0u], x3 = xs[v3 ? c[u].w : 0u];
-            a0 = __builtin_fmaf(v0 ? w[u].x : 0.0f, v0 ? x0 : 0.0f, a0);
-            a1 = __builtin_fmaf(v1 ? w[u].y : 0.0f, v1 ? x1 : 0.0f, a1);
-            a2 = __builtin_fmaf(v2 ? w[u].z : 0.0f, v2 ? x2 : 0.0f, a2);
-            a3 = __builtin_fmaf(v3 ? w[u].w : 0.0f, v3 ? x3 : 0.0f, a3);
-        }
+        RowLoads L;
+        row_issue(Wd4, idx4, beg, end, q0, L);
+        row_consume(L, beg, end, q0, xs, a0, a1, a2, a3);
     }
     return group_sum<64>((a0 + a1) + (a2 + a3));
 }
@@ -102,15 +125,43 @@ void matvec_rows_kernel(const float *__restrict__ Wd, const uint32_t *__restrict
                         const float *__restrict__ bias, float *__restrict__ y)
 {
     extern __shared__ float lds_x[];
-    const float *xs = stage_x<XLDS>(x, n, lds_x);
     const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t wave = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6));
     const uint32_t nwaves = gridDim.x * kWavesPerBlock;
-    for (uint32_t row = wave; row < count; row += nwaves) {
-        const uint64_t beg = (uint64_t)row * r;
-        const float s = wave_row_dot(reinterpret_cast<const f32x4 *>(Wd), reinterpret_cast<const u32x4 *>(idx),
-                                     beg, beg + nnz[row], xs, lane);
+    const f32x4 *Wd4 = reinterpret_cast<const f32x4 *>(Wd);
+    const u32x4 *idx4 = reinterpret_cast<const u32x4 *>(idx);
+    // Rows are pipelined: the first 1024 slots of the next row are requested before the current
+    // row is reduced, and those of the wave's first row before x is staged, so that a wave always
+    // has a row's worth of loads in flight.
+    // Row lengths are fetched two rows ahead, so that requesting a row never waits for its length.
+    uint32_t row = wave;
+    uint64_t beg = (uint64_t)row * r, end = beg + (row < count ? nnz[row] : 0u);
+    uint32_t len1 = row + nwaves < count ? nnz[row + nwaves] : 0u;          // length of the next row
+    RowLoads cur, nxt;
+    if (row < count) row_issue(Wd4, idx4, beg, end, (beg >> 2) + lane, cur);
+    const float *xs = stage_x<XLDS>(x, n, lds_x);
+    for (; row < count; row += nwaves) {
+        const uint32_t nrow = row + nwaves;
+        const uint64_t nbeg = (uint64_t)nrow * r, nend = nbeg + len1;
+        if (nrow < count) row_issue(Wd4, idx4, nbeg, nend, (nbeg >> 2) + lane, nxt);
+        const uint32_t len2 = (uint64_t)nrow + nwaves < count ? nnz[nrow + nwaves] : 0u;
+        float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+        if (end > beg) {
+            const uint64_t qlast = (end - 1) >> 2;
+            uint64_t q0 = (beg >> 2) + lane;
+            row_consume(cur, beg, end, q0, xs, a0, a1, a2, a3);
+            for (q0 += 256; q0 <= qlast; q0 += 256) {            // rows longer than 1024 slots
+                RowLoads more;
+                row_issue(Wd4, idx4, beg, end, q0, more);
+                row_consume(more, beg, end, q0, xs, a0, a1, a2, a3);
+            }
+        }
+        const float s = group_sum<64>((a0 + a1) + (a2 + a3));
         if (lane == 0) y[row] = (bias ? bias[row] : 0.0f) + s;
+        cur = nxt;
+        beg = nbeg;
+        end = nend;
+        len1 = len2;
     }
 }
 
@@ -227,8 +278,9 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
     const uint32_t cus = (uint32_t)ctx->compute_units;
     const size_t lds = (size_t)E->n * sizeof(float);
     if (layout == SO_LAYOUT_ROW) {
-        // Two resident workgroups per compute unit: 32 waves streaming per CU.
-        const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, kWavesPerBlock), 2u * cus));
+        // One resident workgroup per compute unit (the pipelined rows need the registers); each of
+        // its 16 waves keeps two rows' loads in flight.
+        const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, kWavesPerBlock), cus));
         if (use_lds(ctx, matvec_rows_kernel<true>, E->n, E->total_nnz, blocks))
             matvec_rows_kernel<true><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->r,
                                                                            dx, E->n, dBias, dy);
