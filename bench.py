@@ -128,7 +128,38 @@ def cpu_baseline_matmul(E, X, bias, y_gpu, budget_s=15.0):
     }
 
 
-def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup):
+def cpu_baseline_matvec(E, x, b, y_gpu, nbytes):
+    """The same matvec on the host cores: the reference's compiled kernel (which also writes its
+    E.Xt gather buffer, src/ellpack_matvec.cpp:50-52) or the plain-C restatement; 1 warm-up,
+    median of 9."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    from oracle import EllpackArrays, Oracle, Ref
+    Eo = EllpackArrays(E.m, E.n, E.r, E.Wd, E.idx, E.nnz)
+    if Ref.available():
+        ref = Ref()
+        h = ref.from_arrays(Eo)
+        y = np.empty(E.m, dtype=np.float32)
+        run, kind = (lambda: ref.matvec(h, x, b, out=y)), "reference"
+    else:
+        orc, holder = Oracle(), {}
+
+        def run():
+            holder["y"] = orc.matvec(Eo, x, b)
+        kind = "port"
+    run()
+    ts = []
+    for _ in range(9):
+        t0 = time.perf_counter()
+        run()
+        ts.append(time.perf_counter() - t0)
+    ycpu = y if kind == "reference" else holder["y"]
+    med = statistics.median(ts)
+    return {"us_per_call": round(med * 1e6, 1), "GBps": round(nbytes / med / 1e9, 1), "kind": kind,
+            "cores": int(os.environ.get("OMP_NUM_THREADS", len(os.sched_getaffinity(0)))),
+            "gpu_max_rel_err_vs_cpu": float(np.abs(ycpu.astype(np.float64) - y_gpu).max() / max(np.abs(ycpu).max(), 1e-30))}
+
+
+def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup, with_cpu=True):
     E, x, b = gen()
     dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, layouts)
     dx, dB, dy = ctx.array(x), ctx.array(b), ctx.empty((E.m,))
@@ -137,6 +168,8 @@ def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup
     out = {"workload": name, "m": E.m, "n": E.n, "r": E.r, "nnz": E.total_nnz, "us_per_launch": round(ms * 1e3, 2),
            "alg_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1), "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
            "padded_bytes": 8 * E.m * E.r}
+    if with_cpu:
+        out["cpu_baseline"] = cpu_baseline_matvec(E, x, b, dy.download(), nbytes)
     # Cache-cold figure: the streamed arrays (66-108 MB) fit the 256 MB Infinity Cache when the
     # same launch repeats back to back, so also rotate the launches over enough copies of the
     # matrix that a copy has been evicted by the time its turn comes again.
@@ -343,11 +376,11 @@ def main():
         dst.free()
         log("matvec 16384^2 uniform ...")
         extras["matvec_uniform"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 16384x16384, 95% Bernoulli",
-                                                datagen.config2a, hipabi.LAYOUT_ROW, hipabi.LAYOUT_ROW, k, args.warmup)
+                                                datagen.config2a, hipabi.LAYOUT_ROW, hipabi.LAYOUT_ROW, k, args.warmup, not args.no_cpu)
         log("matvec 16384^2 zipf ...")
         extras["matvec_zipf"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048",
                                              datagen.config2b, hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS, hipabi.LAYOUT_BINS,
-                                             k, args.warmup)
+                                             k, args.warmup, not args.no_cpu)
         log("sparse MLP ...")
         extras["mlp"] = bench_mlp(k, args.warmup, with_cpu=not args.no_cpu)
         log("sparse CNN ...")
