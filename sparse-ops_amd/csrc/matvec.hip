@@ -44,7 +44,10 @@ template <bool XLDS>
 __device__ __forceinline__ const float *stage_x(const float *__restrict__ x, uint32_t n, float *lds)
 {
     if (!XLDS) return x;
-    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) lds[i] = x[i];
+    const uint32_t n4 = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) ? n / 4 : 0;     // 16-byte copies when x is aligned
+    for (uint32_t i = threadIdx.x; i < n4; i += blockDim.x)
+        reinterpret_cast<float4 *>(lds)[i] = reinterpret_cast<const float4 *>(x)[i];
+    for (uint32_t i = n4 * 4 + threadIdx.x; i < n; i += blockDim.x) lds[i] = x[i];
     __syncthreads();
     return lds;
 }
