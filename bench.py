@@ -33,6 +33,9 @@ VALU_FP32_PEAK_TF = 157.3    # MI355X vector fp32 (packed FMA); 78.6 with plain 
 # (FETCH_SIZE, WRITE_SIZE) scaled by a plain copy of known size; see the pmc summary
 # under profiles/.  None until measured for the kernel that currently runs.
 MEASURED_TRAFFIC_BYTES = 91_300_000   # ellpack_matmul_tiled_kernel: 87.1 MB fetched + 4.19 MB written
+# the same counters for the two matvec kernels (profiles/bench_all_kernels__pmc_hbm_bytes.txt)
+MEASURED_MATVEC_TRAFFIC = {"ellpack_matvec 16384x16384, 95% Bernoulli": 112_300_000,
+                           "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048": 69_800_000}
 
 
 def log(*a):
@@ -167,7 +170,7 @@ def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup
     nbytes = 8 * E.total_nnz + 4 * E.m + 4 * E.m + 4 * E.n + 4 * E.m
     out = {"workload": name, "m": E.m, "n": E.n, "r": E.r, "nnz": E.total_nnz, "us_per_launch": round(ms * 1e3, 2),
            "alg_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1), "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
-           "padded_bytes": 8 * E.m * E.r}
+           "padded_bytes": 8 * E.m * E.r, "traffic": MEASURED_MATVEC_TRAFFIC.get(name)}
     if with_cpu:
         out["cpu_baseline"] = cpu_baseline_matvec(E, x, b, dy.download(), nbytes)
     # Cache-cold figure: the streamed arrays (66-108 MB) fit the 256 MB Infinity Cache when the
