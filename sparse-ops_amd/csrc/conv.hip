@@ -539,6 +539,25 @@ void conv_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_
 }
 
 
+// Channels per wave for batch `batch`.  Cost of a layer ~ rounds of workgroups over the chip x
+// channels per wave x (fixed + per-wave share of the chunk overhead + per-run overhead), `run`
+// being the mean number of nonzeros per (channel, chunk); constants fitted on MI355X to the 3x3
+// layers of a ResNet-18-shaped stack at batch 32.
+int choose_cpw(const so_ctx *ctx, const so_conv_window &w, uint32_t cout, double run, uint32_t batch)
+{
+    int best = 1, cpw_max = 8;
+    if (const char *e = getenv("SPARSEOPS_CONV_CPW")) cpw_max = atoi(e);
+    double best_cost = 0.0;
+    for (int cpw : {8, 4, 2, 1}) {
+        if (cpw > cpw_max && cpw != 1) continue;
+        const uint64_t wgs = window_workgroups(w, cout, (uint32_t)cpw, batch);
+        const double rounds = (double)so_ceil_div((uint32_t)std::min<uint64_t>(wgs, 1u << 30), (uint32_t)ctx->compute_units);
+        const double cost = rounds * cpw * (6.5 + 10.0 / cpw + 29.0 / run);
+        if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; best = cpw; }
+    }
+    return best;
+}
+
 // Chooses tile, channel chunk and channels per wave for the windowed kernel and uploads its
 // arrays.  Leaves plan->win.cc == 0 when the geometry does not suit the kernel (a chunk must
 // hold enough nonzeros to amortise its copy and barrier; the whole output must give the chip
@@ -585,20 +604,7 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     const double run = nnz_avg / w.nch;
     if (run < 6.0) return SO_OK;
     if ((uint64_t)cc * g.H_in * g.W_in >= (1ull << 24)) return SO_OK;   // int32 offsets up to batch 128
-    // Channels per wave.  Cost of a layer ~ rounds of workgroups over the chip x channels per wave x
-    // (fixed + per-wave share of the chunk overhead + per-run overhead); constants fitted on MI355X
-    // to the 3x3 layers of a ResNet-18-shaped stack at batch 32.
-    w.cpw = 1;
-    int cpw_max = 8;
-    if (const char *e = getenv("SPARSEOPS_CONV_CPW")) cpw_max = atoi(e);
-    double best_cost = 0.0;
-    for (int cpw : {8, 4, 2, 1}) {
-        if (cpw > cpw_max && cpw != 1) continue;
-        const uint64_t wgs = window_workgroups(w, g.Cout, (uint32_t)cpw, batch);
-        const double rounds = (double)so_ceil_div((uint32_t)std::min<uint64_t>(wgs, 1u << 30), (uint32_t)ctx->compute_units);
-        const double cost = rounds * cpw * (6.5 + 10.0 / cpw + 29.0 / run);
-        if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; w.cpw = cpw; }
-    }
+    w.cpw = choose_cpw(ctx, w, g.Cout, run, batch);
     const uint32_t cpw = (uint32_t)w.cpw;
     w.groups = so_ceil_div(E->m, cpw);
 
@@ -751,8 +757,14 @@ extern "C" so_status so_conv_plan_tune(so_ctx *ctx, so_conv_plan *plan, uint32_t
     SO_REQUIRE(ctx && plan, "so_conv_plan_tune: null argument");
     // The layout depends on the batch only through the number of batch tiles.
     const uint32_t batch = std::max(4u, B / 4u * 4u);
-    if (batch == plan->tuned_batch) return SO_OK;
+    if (batch == plan->tuned_batch || plan->win.cc == 0) return SO_OK;
     const so_ellpack *E = plan->E;
+    // Rebuild only if the batch changes the choice of channels per wave.
+    const double run = (double)E->total_nnz / (double)plan->g.Cout / plan->win.nch;
+    if (choose_cpw(ctx, plan->win, plan->g.Cout, run, batch) == plan->win.cpw) {
+        plan->tuned_batch = batch;
+        return SO_OK;
+    }
     const size_t slots = (size_t)E->m * E->r;
     std::vector<uint32_t> idx(slots), nnz(E->m);
     std::vector<float> Wd(slots);
