@@ -128,6 +128,10 @@ so_status so_ellpack_dims(const so_ellpack *E, uint32_t *m, uint32_t *n, uint32_
 so_status so_ellpack_download(so_ctx *ctx, const so_ellpack *E, int layout,
                               float *Wd, uint32_t *idx, uint32_t *nnz);
 
+/* decode_from_ellpack (src/ellpack_encoder.cpp:46-60) on the device: dDense [m x n] row-major
+ * is zeroed, then the first nnz[i] entries of every row are scattered into it. */
+so_status so_ellpack_decode(so_ctx *ctx, const so_ellpack *E, float *dDense);
+
 /* ---- kernels ------------------------------------------------------------ */
 
 /* Y[m x C] = act(E * X[n x C] + bias): ellpack_matmul_fused<USE_MASK,FUSE_RELU>

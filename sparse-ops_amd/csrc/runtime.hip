@@ -441,6 +441,41 @@ extern "C" so_status so_ellpack_dims(const so_ellpack *E, uint32_t *m, uint32_t 
     return SO_OK;
 }
 
+namespace {
+
+// One wave per row: its stored nonzeros go to their columns (ascending, distinct, so no two
+// lanes write the same element).
+__global__ __launch_bounds__(256)
+void ellpack_decode_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
+                           const uint32_t *__restrict__ nnz, uint32_t m, uint32_t n, uint32_t r,
+                           float *__restrict__ W)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t nwaves = gridDim.x * 4u;
+    for (uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6); row < m; row += nwaves) {
+        const uint32_t cnt = nnz[row];
+        for (uint32_t k = lane; k < cnt; k += 64u)
+            W[(size_t)row * n + idx[(size_t)row * r + k]] = Wd[(size_t)row * r + k];
+    }
+}
+
+} // namespace
+
+extern "C" so_status so_ellpack_decode(so_ctx *ctx, const so_ellpack *E, float *dDense)
+{
+    SO_REQUIRE(ctx && E, "so_ellpack_decode: null argument");
+    const size_t total = (size_t)E->m * E->n;
+    if (total == 0) return SO_OK;
+    SO_REQUIRE(dDense != nullptr, "so_ellpack_decode: null output");
+    so_status s = so_fill_zero(ctx, dDense, total * sizeof(float));
+    if (s != SO_OK) return s;
+    if (E->r == 0) return SO_OK;
+    const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, 4u), 16u * (uint32_t)ctx->compute_units));
+    ellpack_decode_kernel<<<blocks, 256, 0, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->n, E->r, dDense);
+    SO_LAUNCH_CHECK();
+    return SO_OK;
+}
+
 extern "C" so_status so_ellpack_download(so_ctx *ctx, const so_ellpack *E, int layout,
                                          float *Wd, uint32_t *idx, uint32_t *nnz)
 {

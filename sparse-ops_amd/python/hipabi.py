@@ -19,7 +19,7 @@ LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS, LAYOUT_TILED = 1, 2, 4, 8
 SYMBOLS = (
     "so_device_count so_init so_destroy so_last_error so_device_info so_malloc so_free so_h2d so_d2h "
     "so_d2d so_fill_zero so_sync so_timer_begin so_timer_end so_ellpack_upload so_ellpack_free "
-    "so_ellpack_dims so_ellpack_download so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
+    "so_ellpack_dims so_ellpack_download so_ellpack_decode so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
     "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_graph_begin so_graph_end "
     "so_graph_launch so_graph_free").split()
 
@@ -75,6 +75,7 @@ def load_library(path=None):
         "so_ellpack_dims": [_vp, ct.POINTER(_u32), ct.POINTER(_u32), ct.POINTER(_u32),
                             ct.POINTER(ct.c_uint64), ct.POINTER(ct.c_int)],
         "so_ellpack_download": [_vp, _vp, ct.c_int, _vp, _vp, _vp],
+        "so_ellpack_decode": [_vp, _vp, _vp],
         "so_matmul": [_vp, _vp, _vp, _u32, _vp, _vp, ct.c_int],
         "so_matvec": [_vp, _vp, _vp, _vp, _vp, ct.c_int],
         "so_conv_plan_create": [_vp, _vp, ct.POINTER(ConvGeom), ct.POINTER(_vp)],
@@ -134,6 +135,14 @@ class DeviceArray:
 class DeviceEllpack:
     def __init__(self, ctx, handle, m, n, r):
         self.ctx, self.h, self.m, self.n, self.r = ctx, handle, m, n, r
+
+    def decode(self):
+        """-> the dense (m, n) matrix, decoded on the device."""
+        dW = self.ctx.empty((self.m, self.n))
+        self.ctx._ck(self.ctx.lib.so_ellpack_decode(self.ctx.h, self.h, dW.ptr))
+        W = dW.download()
+        dW.free()
+        return W
 
     def download(self, layout=LAYOUT_ROW):
         shape = (self.m, self.r) if layout == LAYOUT_ROW else (self.r, self.m)

@@ -237,3 +237,27 @@ def test_backend_matmul(backend, oracle, m, n, C, sp):
         assert np.array_equal(backend.ellpack_matmul(E, X, None), oracle.matmul(oracle.encode(W), X, None))
         # non-contiguous / float64 inputs are force-cast like the reference does (src/bindings.cpp:112-113)
         assert np.array_equal(backend.ellpack_matmul(E, np.asfortranarray(X).astype(np.float64), b), y)
+
+
+@pytest.mark.parametrize("m,n,sp", [(1, 1, 0.), (7, 130, .6), (300, 257, .9), (64, 1000, .99), (5, 9, 1.)])
+def test_device_decode_round_trip(ctx, oracle, golden, m, n, sp):
+    """so_ellpack_decode == decode_from_ellpack: exact round trip of the encoder (the reference's
+    own encoder test, tests/unit/test_ellpack_encoder.py), -0.0 dropped, NaN kept."""
+    rng = np.random.default_rng(m * 13 + n)
+    W = sparse_matrix(rng, m, n, sp)
+    if m > 4:
+        W[2, 1] = np.nan
+        W[3, 0] = -0.0
+    E = datagen.encode_dense(W)
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+    D = dE.decode()
+    dE.free()
+    want = oracle.decode(as_oracle(E))
+    assert D.shape == (m, n) and np.array_equal(D, want, equal_nan=True)
+    assert np.array_equal(np.signbit(D), np.signbit(want))          # the dropped -0.0 comes back as +0.0
+    assert np.array_equal(D, np.where(W == 0, 0, W), equal_nan=True)
+    # the committed reference vectors decode to the reference's own dense matrix
+    Eg = datagen.encode_dense(golden["enc_W"])
+    dEg = ctx.upload_ellpack(Eg.Wd, Eg.idx, Eg.nnz, Eg.m, Eg.n, Eg.r)
+    assert np.array_equal(dEg.decode(), golden["enc_W"] + 0.0)
+    dEg.free()
