@@ -128,6 +128,12 @@ so_status so_ellpack_dims(const so_ellpack *E, uint32_t *m, uint32_t *n, uint32_
 so_status so_ellpack_download(so_ctx *ctx, const so_ellpack *E, int layout,
                               float *Wd, uint32_t *idx, uint32_t *nnz);
 
+/* convert_to_ellpack (src/ellpack_encoder.cpp:6-44) on the device: dDense is a row-major
+ * [m x n] fp32 matrix in device memory; the handle holds the ROW layout with the same
+ * contents the host encoder produces (per row the entries with v != 0.0f in ascending
+ * column order, so -0.0f is dropped and NaN kept; r = longest row; zero padding).
+ * Other layouts: download and upload again with the layouts wanted. */
+so_status so_ellpack_encode(so_ctx *ctx, const float *dDense, uint32_t m, uint32_t n, so_ellpack **out);
 /* decode_from_ellpack (src/ellpack_encoder.cpp:46-60) on the device: dDense [m x n] row-major
  * is zeroed, then the first nnz[i] entries of every row are scattered into it. */
 so_status so_ellpack_decode(so_ctx *ctx, const so_ellpack *E, float *dDense);

@@ -461,6 +461,93 @@ void ellpack_decode_kernel(const float *__restrict__ Wd, const uint32_t *__restr
 
 } // namespace
 
+namespace {
+
+// Pass 1 of the encoder: one wave per row counts the entries with v != 0.0f.
+__global__ __launch_bounds__(256)
+void ellpack_count_kernel(const float *__restrict__ W, uint32_t m, uint32_t n, uint32_t *__restrict__ nnz)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t nwaves = gridDim.x * 4u;
+    for (uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6); row < m; row += nwaves) {
+        const float *wr = W + (size_t)row * n;
+        uint32_t c = 0;
+        for (uint32_t j = lane; j < n; j += 64u) c += wr[j] != 0.0f ? 1u : 0u;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
+        if (lane == 0) nnz[row] = c;
+    }
+}
+
+// Pass 2: one wave per row packs (value, column) in ascending column order.  For each group of
+// 64 columns the lanes that hold a nonzero get consecutive slots (a prefix count over the wave's
+// ballot), so the order inside the row is the column order.  Wd/idx were zero-filled before.
+__global__ __launch_bounds__(256)
+void ellpack_pack_kernel(const float *__restrict__ W, uint32_t m, uint32_t n, uint32_t r,
+                         float *__restrict__ Wd, uint32_t *__restrict__ idx)
+{
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t nwaves = gridDim.x * 4u;
+    for (uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6); row < m; row += nwaves) {
+        const float *wr = W + (size_t)row * n;
+        uint32_t base = 0;
+        for (uint32_t j0 = 0; j0 < n; j0 += 64u) {
+            const uint32_t j = j0 + lane;
+            const float v = j < n ? wr[j] : 0.0f;
+            const bool keep = v != 0.0f;
+            const uint64_t mask = __ballot(keep);
+            if (keep) {
+                const uint32_t pos = base + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+                Wd[(size_t)row * r + pos] = v;
+                idx[(size_t)row * r + pos] = j;
+            }
+            base += (uint32_t)__popcll(mask);
+        }
+    }
+}
+
+} // namespace
+
+extern "C" so_status so_ellpack_encode(so_ctx *ctx, const float *dDense, uint32_t m, uint32_t n, so_ellpack **out)
+{
+    SO_REQUIRE(ctx && out, "so_ellpack_encode: null argument");
+    *out = nullptr;
+    SO_REQUIRE(dDense != nullptr || (uint64_t)m * n == 0, "so_ellpack_encode: null matrix");
+    so_ellpack *E = new (std::nothrow) so_ellpack();
+    if (!E) { so_set_error("so_ellpack_encode: host allocation failed"); return SO_ERR_OOM; }
+    E->m = m; E->n = n;
+    E->layouts = SO_LAYOUT_ROW;
+    std::vector<uint32_t> nnz(m, 0);
+    void *p = nullptr;
+    so_status s = so_malloc(ctx, (size_t)m * sizeof(uint32_t) + 16, &p);
+    if (s == SO_OK) { E->d_nnz = (uint32_t *)p; s = so_fill_zero(ctx, p, (size_t)m * sizeof(uint32_t) + 16); }
+    const uint32_t blocks = std::max(1u, std::min(so_ceil_div(m, 4u), 16u * (uint32_t)ctx->compute_units));
+    if (s == SO_OK && m && n) {
+        ellpack_count_kernel<<<blocks, 256, 0, ctx->stream>>>(dDense, m, n, E->d_nnz);
+        if (hipGetLastError() != hipSuccess) { so_set_error("so_ellpack_encode: launch failed"); s = SO_ERR_HIP; }
+    }
+    if (s == SO_OK && m) s = so_d2h(ctx, nnz.data(), E->d_nnz, (size_t)m * sizeof(uint32_t));
+    if (s == SO_OK) {
+        for (uint32_t c : nnz) { E->total_nnz += c; E->max_nnz = std::max(E->max_nnz, c); }
+        E->r = E->max_nnz;                               // r = longest row (src/ellpack_encoder.cpp:10-17)
+        const size_t bytes = (size_t)m * E->r * sizeof(float) + 16;
+        s = so_malloc(ctx, bytes, &p);
+        if (s == SO_OK) { E->d_Wd = (float *)p; s = so_fill_zero(ctx, p, bytes); }
+        if (s == SO_OK) s = so_malloc(ctx, bytes, &p);
+        if (s == SO_OK) { E->d_idx = (uint32_t *)p; s = so_fill_zero(ctx, p, bytes); }
+    }
+    if (s == SO_OK && E->r) {
+        ellpack_pack_kernel<<<blocks, 256, 0, ctx->stream>>>(dDense, m, n, E->r, E->d_Wd, E->d_idx);
+        if (hipGetLastError() != hipSuccess) { so_set_error("so_ellpack_encode: launch failed"); s = SO_ERR_HIP; }
+    }
+    if (s != SO_OK) {
+        (void)so_ellpack_free(ctx, E);
+        return s;
+    }
+    *out = E;
+    return SO_OK;
+}
+
 extern "C" so_status so_ellpack_decode(so_ctx *ctx, const so_ellpack *E, float *dDense)
 {
     SO_REQUIRE(ctx && E, "so_ellpack_decode: null argument");

@@ -19,7 +19,7 @@ LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS, LAYOUT_TILED = 1, 2, 4, 8
 SYMBOLS = (
     "so_device_count so_init so_destroy so_last_error so_device_info so_malloc so_free so_h2d so_d2h "
     "so_d2d so_fill_zero so_sync so_timer_begin so_timer_end so_ellpack_upload so_ellpack_free "
-    "so_ellpack_dims so_ellpack_download so_ellpack_decode so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
+    "so_ellpack_dims so_ellpack_download so_ellpack_decode so_ellpack_encode so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
     "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_graph_begin so_graph_end "
     "so_graph_launch so_graph_free").split()
 
@@ -76,6 +76,7 @@ def load_library(path=None):
                             ct.POINTER(ct.c_uint64), ct.POINTER(ct.c_int)],
         "so_ellpack_download": [_vp, _vp, ct.c_int, _vp, _vp, _vp],
         "so_ellpack_decode": [_vp, _vp, _vp],
+        "so_ellpack_encode": [_vp, _vp, _u32, _u32, ct.POINTER(_vp)],
         "so_matmul": [_vp, _vp, _vp, _u32, _vp, _vp, ct.c_int],
         "so_matvec": [_vp, _vp, _vp, _vp, _vp, ct.c_int],
         "so_conv_plan_create": [_vp, _vp, ct.POINTER(ConvGeom), ct.POINTER(_vp)],
@@ -208,6 +209,14 @@ class Context:
         h = _vp()
         self._ck(self.lib.so_ellpack_upload(self.h, _ptr(Wd), _ptr(idx), _ptr(nnz), m, n, r, layouts, ct.byref(h)))
         return DeviceEllpack(self, h.value, m, n, r)
+
+    def encode_dense(self, dW, m, n):
+        """Device-side convert_to_ellpack of the (m, n) fp32 DeviceArray dW -> DeviceEllpack (ROW layout)."""
+        h = _vp()
+        self._ck(self.lib.so_ellpack_encode(self.h, dW.ptr if dW is not None else None, m, n, ct.byref(h)))
+        r = ct.c_uint32()
+        self._ck(self.lib.so_ellpack_dims(h, None, None, ct.byref(r), None, None))
+        return DeviceEllpack(self, h.value, m, n, r.value)
 
     def matmul(self, E, dX, C, dBias, dY, act="none"):
         self._ck(self.lib.so_matmul(self.h, E.h, dX.ptr, C, dBias.ptr if dBias else None, dY.ptr, ACT[act]))

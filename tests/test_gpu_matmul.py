@@ -261,3 +261,49 @@ def test_device_decode_round_trip(ctx, oracle, golden, m, n, sp):
     dEg = ctx.upload_ellpack(Eg.Wd, Eg.idx, Eg.nnz, Eg.m, Eg.n, Eg.r)
     assert np.array_equal(dEg.decode(), golden["enc_W"] + 0.0)
     dEg.free()
+
+
+@pytest.mark.parametrize("m,n,sp", [(1, 1, 0.), (7, 130, .6), (300, 257, .9), (64, 1000, .99), (5, 9, 1.), (33, 64, .5),
+                                    (1024, 1024, .9)])
+def test_device_encoder_matches_host_encoder(ctx, oracle, m, n, sp):
+    """so_ellpack_encode == convert_to_ellpack bit for bit (nnz, r, idx, Wd, zero padding; -0.0
+    dropped, NaN kept), and the encoded matrix multiplies like the host-encoded one."""
+    rng = np.random.default_rng(m * 17 + n)
+    W = sparse_matrix(rng, m, n, sp)
+    if m > 4:
+        W[2, 1] = np.nan
+        W[3, 0] = -0.0
+        W[4] = 0
+    E = datagen.encode_dense(W)
+    dW = ctx.array(W)
+    dE = ctx.encode_dense(dW, m, n)
+    assert dE.r == E.r
+    Wd, idx, nnz = dE.download()
+    assert np.array_equal(nnz, E.nnz) and np.array_equal(idx, E.idx.reshape(m, E.r))
+    assert np.array_equal(Wd.view(np.uint32), E.Wd.reshape(m, E.r).view(np.uint32))        # bits, NaN included
+    assert np.array_equal(dE.decode(), oracle.decode(as_oracle(E)), equal_nan=True)
+    if m > 4:
+        W[2, 1] = 1.5                                     # no NaN for the product check
+        dW2 = ctx.array(W)
+        dE2 = ctx.encode_dense(dW2, m, n)
+        X = rng.standard_normal((n, 8)).astype(np.float32)
+        dX, dY = ctx.array(X), ctx.empty((m, 8))
+        ctx.matmul(dE2, dX, 8, None, dY, "none")
+        assert np.array_equal(dY.download(), oracle.matmul(as_oracle(datagen.encode_dense(W)), X, None))
+        for a in (dW2, dX, dY):
+            a.free()
+        dE2.free()
+    dW.free()
+    dE.free()
+
+
+def test_device_encoder_degenerate(ctx):
+    for (m, n) in [(0, 0), (0, 5), (5, 0)]:
+        dE = ctx.encode_dense(None, m, n)
+        assert dE.r == 0
+        dE.free()
+    dZ = ctx.array(np.zeros((6, 70), np.float32))
+    dE = ctx.encode_dense(dZ, 6, 70)
+    assert dE.r == 0 and np.array_equal(dE.decode(), np.zeros((6, 70), np.float32))
+    dZ.free()
+    dE.free()
