@@ -44,8 +44,13 @@ __global__ __launch_bounds__(kBlock)
 void maxpool4_kernel(so_pool_geom p, const float *__restrict__ X, uint32_t B4, uint32_t total,
                      float *__restrict__ Y)
 {
-    const uint32_t stride = gridDim.x * kBlock;
-    for (uint32_t q = blockIdx.x * kBlock + threadIdx.x; q < total; q += stride) {
+    // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one contiguous eighth of the
+    // output instead, so that the input rows two neighbouring output rows share meet in one L2.
+    const uint32_t per_xcd = gridDim.x / 8u;                     // the grid is a multiple of 8
+    const uint32_t vblock = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    const uint32_t chunk = (total + 8u * per_xcd - 1u) / (8u * per_xcd);        // outputs per workgroup
+    const uint32_t q_end = min(total, (vblock + 1u) * chunk);
+    for (uint32_t q = vblock * chunk + threadIdx.x; q < q_end; q += kBlock) {
         const uint32_t b = q % B4;
         uint32_t t = q / B4;
         const uint32_t wo = t % p.W_out; t /= p.W_out;
@@ -150,7 +155,7 @@ extern "C" so_status so_maxpool(so_ctx *ctx, const so_pool_geom *p, const float 
                "so_maxpool: output size does not fit the input");
     if (B % 4 == 0 && (((uintptr_t)dX | (uintptr_t)dY) & 15) == 0 && total / 4 < (1ull << 31) &&
         (uint64_t)p->H * p->W * (B / 4) < (1ull << 31))
-        maxpool4_kernel<<<blocks_for(ctx, total / 4), kBlock, 0, ctx->stream>>>(*p, dX, B / 4, (uint32_t)(total / 4), dY);
+        maxpool4_kernel<<<(blocks_for(ctx, total / 4) + 7u) / 8u * 8u, kBlock, 0, ctx->stream>>>(*p, dX, B / 4, (uint32_t)(total / 4), dY);   // a multiple of 8: the kernel deals whole eighths to the XCDs
     else
         maxpool_kernel<<<blocks_for(ctx, total), kBlock, 0, ctx->stream>>>(*p, dX, B, total, dY);
     SO_LAUNCH_CHECK();
