@@ -22,6 +22,7 @@
 #include "so_internal.h"
 
 #include <algorithm>
+#include <cstdlib>
 
 namespace {
 
@@ -62,18 +63,21 @@ struct RowLoads {
     u32x4 c[4];
 };
 
+// G = lanes that share a row (64, 32, 16 or 8): a pass of the row covers 16 G slots.
+template <int G = 64>
 __device__ __forceinline__ void row_issue(const f32x4 *__restrict__ Wd4, const u32x4 *__restrict__ idx4,
                                           uint64_t beg, uint64_t end, uint64_t q0, RowLoads &L)
 {
     const uint64_t qlast = end > beg ? (end - 1) >> 2 : beg >> 2;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-        const uint64_t q = std::min<uint64_t>(q0 + 64u * u, qlast);
+        const uint64_t q = std::min<uint64_t>(q0 + (uint64_t)G * u, qlast);
         L.w[u] = __builtin_nontemporal_load(Wd4 + q);
         L.c[u] = __builtin_nontemporal_load(idx4 + q);
     }
 }
 
+template <int G = 64>
 __device__ __forceinline__ void row_consume(const RowLoads &L, uint64_t beg, uint64_t end, uint64_t q0, const float *xs,
                                             float &a0, float &a1, float &a2, float &a3)
 {
@@ -83,7 +87,7 @@ __device__ __forceinline__ void row_consume(const RowLoads &L, uint64_t beg, uin
     const int32_t rel0 = (int32_t)(int64_t)((q0 << 2) - beg);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-        const int32_t rel = rel0 + 256 * u;
+        const int32_t rel = rel0 + 4 * G * u;
         const bool v0 = (uint32_t)rel < len, v1 = (uint32_t)(rel + 1) < len;
         const bool v2 = (uint32_t)(rel + 2) < len, v3 = (uint32_t)(rel + 3) < len;
         const float x0 = xs[v0 ? L.c[u].x : 0u], x1 = xs[v1 ? L.c[u].y : 0u];
@@ -119,8 +123,9 @@ __device__ __forceinline__ float group_row_dot(const float *__restrict__ Wd, con
     return group_sum<G>(a);
 }
 
-// rows == nullptr: row ids are 0..count-1; otherwise the ids come from the list.
-template <bool XLDS>
+// G lanes per row: a wave works on 64/G rows at a time (whole waves for rows longer than 512
+// slots, a half, a quarter or an eighth of a wave for shorter ones, so that short rows do not leave lanes idle).
+template <bool XLDS, int G>
 __global__ __launch_bounds__(kBlock)
 void matvec_rows_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
                         const uint32_t *__restrict__ nnz, uint32_t count, uint32_t r,
@@ -128,39 +133,41 @@ void matvec_rows_kernel(const float *__restrict__ Wd, const uint32_t *__restrict
                         const float *__restrict__ bias, float *__restrict__ y)
 {
     extern __shared__ float lds_x[];
-    const uint32_t lane = threadIdx.x & 63u;
+    constexpr uint32_t RPW = 64 / G;                                     // rows per wave
+    const uint32_t lane = threadIdx.x & 63u, sub = lane % G, grp = lane / G;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6));
-    const uint32_t nwaves = gridDim.x * kWavesPerBlock;
+    const uint32_t stride = gridDim.x * kWavesPerBlock * RPW;            // rows between a group's consecutive rows
     const f32x4 *Wd4 = reinterpret_cast<const f32x4 *>(Wd);
     const u32x4 *idx4 = reinterpret_cast<const u32x4 *>(idx);
-    // Rows are pipelined: the first 1024 slots of the next row are requested before the current
-    // row is reduced, and those of the wave's first row before x is staged, so that a wave always
-    // has a row's worth of loads in flight.
-    // Row lengths are fetched two rows ahead, so that requesting a row never waits for its length.
-    uint32_t row = wave;
+    // Rows are pipelined: the first 16 G slots of the next row are requested before the current
+    // row is reduced, and those of the group's first row before x is staged, so that a wave always
+    // has a row's worth of loads in flight.  Row lengths are fetched two rows ahead, so that
+    // requesting a row never waits for its length.
+    uint32_t row = wave * RPW + grp;
     uint64_t beg = (uint64_t)row * r, end = beg + (row < count ? nnz[row] : 0u);
-    uint32_t len1 = row + nwaves < count ? nnz[row + nwaves] : 0u;          // length of the next row
+    uint32_t len1 = (uint64_t)row + stride < count ? nnz[row + stride] : 0u;          // length of the next row
     RowLoads cur, nxt;
-    if (row < count) row_issue(Wd4, idx4, beg, end, (beg >> 2) + lane, cur);
+    if (row < count) row_issue<G>(Wd4, idx4, beg, end, (beg >> 2) + sub, cur);
     const float *xs = stage_x<XLDS>(x, n, lds_x);
-    for (; row < count; row += nwaves) {
-        const uint32_t nrow = row + nwaves;
-        const uint64_t nbeg = (uint64_t)nrow * r, nend = nbeg + len1;
-        if (nrow < count) row_issue(Wd4, idx4, nbeg, nend, (nbeg >> 2) + lane, nxt);
-        const uint32_t len2 = (uint64_t)nrow + nwaves < count ? nnz[nrow + nwaves] : 0u;
+    // all groups of a wave make the same number of trips (the reductions need every lane)
+    for (uint32_t base = wave * RPW; base < count; base += stride, row += stride) {
+        const uint64_t nrow = (uint64_t)row + stride;
+        const uint64_t nbeg = nrow * r, nend = nbeg + len1;
+        if (nrow < count) row_issue<G>(Wd4, idx4, nbeg, nend, (nbeg >> 2) + sub, nxt);
+        const uint32_t len2 = nrow + stride < count ? nnz[nrow + stride] : 0u;
         float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
-        if (end > beg) {
+        if (row < count && end > beg) {
             const uint64_t qlast = (end - 1) >> 2;
-            uint64_t q0 = (beg >> 2) + lane;
-            row_consume(cur, beg, end, q0, xs, a0, a1, a2, a3);
-            for (q0 += 256; q0 <= qlast; q0 += 256) {            // rows longer than 1024 slots
+            uint64_t q0 = (beg >> 2) + sub;
+            row_consume<G>(cur, beg, end, q0, xs, a0, a1, a2, a3);
+            for (q0 += 4 * G; q0 <= qlast; q0 += 4 * G) {        // rows longer than one pass
                 RowLoads more;
-                row_issue(Wd4, idx4, beg, end, q0, more);
-                row_consume(more, beg, end, q0, xs, a0, a1, a2, a3);
+                row_issue<G>(Wd4, idx4, beg, end, q0, more);
+                row_consume<G>(more, beg, end, q0, xs, a0, a1, a2, a3);
             }
         }
-        const float s = group_sum<64>((a0 + a1) + (a2 + a3));
-        if (lane == 0) y[row] = (bias ? bias[row] : 0.0f) + s;
+        const float s = group_sum<G>((a0 + a1) + (a2 + a3));
+        if (sub == 0 && row < count) y[row] = (bias ? bias[row] : 0.0f) + s;
         cur = nxt;
         beg = nbeg;
         end = nend;
@@ -281,15 +288,32 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
     const uint32_t cus = (uint32_t)ctx->compute_units;
     const size_t lds = (size_t)E->n * sizeof(float);
     if (layout == SO_LAYOUT_ROW) {
+        // Lanes per row by the longest row (one pass of 16 G slots should cover it), but never so
+        // few that compute units are left without rows.
+        uint32_t G = E->max_nnz <= 128 ? 8u : E->max_nnz <= 256 ? 16u : E->max_nnz <= 512 ? 32u : 64u;
+        if (const char *e = getenv("SPARSEOPS_MATVEC_LANES")) {
+            const int v = atoi(e);
+            if (v == 8 || v == 16 || v == 32 || v == 64) G = (uint32_t)v;
+        } else {
+            while (G < 64 && so_ceil_div(E->m, kWavesPerBlock * (64u / G)) < cus) G *= 2;
+        }
         // One resident workgroup per compute unit (the pipelined rows need the registers); each of
-        // its 16 waves keeps two rows' loads in flight.
-        const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, kWavesPerBlock), cus));
-        if (use_lds(ctx, matvec_rows_kernel<true>, E->n, E->total_nnz, blocks))
-            matvec_rows_kernel<true><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->r,
-                                                                           dx, E->n, dBias, dy);
-        else
-            matvec_rows_kernel<false><<<blocks, kBlock, 0, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->r,
-                                                                          dx, E->n, dBias, dy);
+        // its 16 waves keeps two passes' loads in flight.
+        const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, kWavesPerBlock * (64u / G)), cus));
+#define SO_MV_ROWS(G)                                                                                              \
+        do {                                                                                                       \
+            if (use_lds(ctx, matvec_rows_kernel<true, G>, E->n, E->total_nnz, blocks))                             \
+                matvec_rows_kernel<true, G><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->r, \
+                                                                                  dx, E->n, dBias, dy);            \
+            else                                                                                                   \
+                matvec_rows_kernel<false, G><<<blocks, kBlock, 0, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->r,  \
+                                                                                 dx, E->n, dBias, dy);             \
+        } while (0)
+        if (G == 8) SO_MV_ROWS(8);
+        else if (G == 16) SO_MV_ROWS(16);
+        else if (G == 32) SO_MV_ROWS(32);
+        else SO_MV_ROWS(64);
+#undef SO_MV_ROWS
     } else if (layout == SO_LAYOUT_SLOT) {
         const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, kBlock), 2u * cus));
         if (use_lds(ctx, matvec_slot_kernel<true>, E->n, E->total_nnz, blocks))

@@ -68,6 +68,33 @@ def test_matvec_every_row_written_once(ctx):
         assert rel_err(y, W @ x) <= TOL, lay
 
 
+@pytest.mark.parametrize("lanes", [8, 16, 32, 64])
+@pytest.mark.parametrize("m,n,kmax", [(3001, 1000, 203), (517, 4099, 700), (64, 300, 17), (70000, 256, 40)])
+def test_matvec_rows_lanes_per_row(ctx, monkeypatch, lanes, m, n, kmax):
+    """The row kernel shares a row among 8, 16, 32 or 64 lanes (picked by the longest row and the
+    row count; forced here): ragged rows including empty ones, odd r, rows longer than one pass."""
+    rng = np.random.default_rng(lanes + m)
+    counts = rng.integers(0, kmax + 1, size=m)
+    counts[::7] = 0
+    counts[1] = kmax
+    cols = [np.sort(rng.choice(n, size=k, replace=False)).astype(np.uint32) for k in counts]
+    vals = [rng.standard_normal(k).astype(np.float32) for k in counts]
+    E = datagen.rows_to_ellpack(m, n, cols, vals)
+    assert E.r == kmax
+    x = rng.standard_normal(n).astype(np.float32)
+    b = rng.standard_normal(m).astype(np.float32)
+    y64 = b.astype(np.float64)
+    for i in range(m):
+        y64[i] += vals[i].astype(np.float64) @ x[cols[i]]
+    monkeypatch.setenv("SPARSEOPS_MATVEC_LANES", str(lanes))
+    y = gpu_matvec(ctx, E, x, b, layouts=hipabi.LAYOUT_ROW, which=(hipabi.LAYOUT_ROW,))[hipabi.LAYOUT_ROW]
+    assert np.isfinite(y).all()
+    assert rel_err(y, y64) <= TOL
+    monkeypatch.delenv("SPARSEOPS_MATVEC_LANES")
+    y_auto = gpu_matvec(ctx, E, x, b, layouts=hipabi.LAYOUT_ROW, which=(hipabi.LAYOUT_ROW,))[hipabi.LAYOUT_ROW]
+    assert rel_err(y_auto, y64) <= TOL
+
+
 def test_matvec_reference_vectors(ctx, golden):
     E = datagen.encode_dense(golden["enc_W"])
     for lay, y in gpu_matvec(ctx, E, golden["mv_x"], golden["mm_bias"]).items():
