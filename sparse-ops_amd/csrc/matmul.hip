@@ -227,6 +227,12 @@ __device__ __forceinline__ uint32_t bcast_u(uint32_t v)
     return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x150 + N, 0xf, 0xf, true);
 }
 
+template <int N>
+__device__ __forceinline__ void fmac_bcast(float &acc, float ew, float x)
+{
+    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(ew), "v"(x), "n"(N));
+}
+
 // Steps N..END-1 of a chunk: all LDS reads first, then the FMAs in step order.
 template <int N, int END>
 struct StepRange {
@@ -237,11 +243,12 @@ struct StepRange {
     }
     static __device__ __forceinline__ void fma(float ew, const float4 *x, float (&acc)[4])
     {
-        const float w = bcast_f<N>(ew);
-        acc[0] = __builtin_fmaf(w, x[0].x, acc[0]);
-        acc[1] = __builtin_fmaf(w, x[0].y, acc[1]);
-        acc[2] = __builtin_fmaf(w, x[0].z, acc[2]);
-        acc[3] = __builtin_fmaf(w, x[0].w, acc[3]);
+        // acc += bcast(ew) * x with the broadcast folded into the multiply-add's first operand
+        // (v_fmac_f32 is a fused multiply-add: one rounding, like fmaf)
+        fmac_bcast<N>(acc[0], ew, x[0].x);
+        fmac_bcast<N>(acc[1], ew, x[0].y);
+        fmac_bcast<N>(acc[2], ew, x[0].z);
+        fmac_bcast<N>(acc[3], ew, x[0].w);
         StepRange<N + 1, END>::fma(ew, x + 1, acc);
     }
 };
@@ -256,6 +263,9 @@ __device__ __forceinline__ void tiled_steps(const char *base, float ew, uint32_t
 {
     float4 x[CNT];
     StepRange<N0, N0 + CNT>::read(base, eoff, x);
+    // a DPP operand must not be read within two cycles of a vector write to it, nor within five of
+    // a vector write to the execution mask; the compiler does not see inside the asm
+    asm volatile("s_nop 4" : "+v"(ew));
     StepRange<N0, N0 + CNT>::fma(ew, x, acc);
 }
 
