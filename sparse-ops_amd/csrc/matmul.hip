@@ -320,7 +320,14 @@ void ellpack_matmul_tiled_kernel(const so_tile_entry *__restrict__ entries, cons
     const bool lcol_ok = c0 + lc * 4 < C;            // C is a multiple of 4
     const float *xsrc = X + (size_t)lr * C + c0 + lc * 4;
     float4 pre[4];
+    const bool slab_full = c0 + so_tiled::kSlabCols <= C;       // wave-uniform
     auto gload = [&](uint32_t t) {
+        if (slab_full && (t + 1) * KT <= n) {                    // whole tile inside X: no per-lane tests
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                pre[i] = *reinterpret_cast<const float4 *>(xsrc + (size_t)(t * KT + 64 * i) * C);
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t xr = t * KT + lr + 64 * i;
