@@ -95,6 +95,10 @@ so_status so_destroy(so_ctx *ctx);
 const char *so_last_error(void);
 /* Device name and compute-unit count of the context's device. */
 so_status so_device_info(so_ctx *ctx, char *name, size_t name_len, int *compute_units);
+/* The SPARSEOPS_* tuning overrides (kernel and layout choices: for tuning and tests, results never
+ * depend on them) are read from the environment by so_init, not per launch as the reference reads
+ * its thread count (src/ellpack_matmul.cpp:21); this reads them again for `ctx`. */
+so_status so_tuning_reload(so_ctx *ctx);
 
 so_status so_malloc(so_ctx *ctx, size_t bytes, void **dptr);
 so_status so_free(so_ctx *ctx, void *dptr);

@@ -546,7 +546,7 @@ void conv_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_
 int choose_cpw(const so_ctx *ctx, const so_conv_window &w, uint32_t cout, double run, uint32_t batch)
 {
     int best = 1, cpw_max = 8;
-    if (const char *e = getenv("SPARSEOPS_CONV_CPW")) cpw_max = atoi(e);
+    if (ctx->tune.conv_cpw > 0) cpw_max = ctx->tune.conv_cpw;
     double best_cost = 0.0;
     for (int cpw : {8, 4, 2, 1}) {
         if (cpw > cpw_max && cpw != 1) continue;
@@ -576,7 +576,7 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     // smaller window lets a chunk hold more channels and the extra tiles give the chip more workgroups
     // (measured: 14 x 14 layer 79 -> 71 us, 7 x 7 layer 89 -> 81 us; 28 x 28 and 56 x 56 lose 8-25 %).
     uint32_t max_px = (uint64_t)g.H_out * g.W_out <= 256 ? 16u : 32u;
-    if (const char *e = getenv("SPARSEOPS_CONV_TILEPX")) max_px = std::max(1, atoi(e));
+    if (ctx->tune.conv_tilepx > 0) max_px = (uint32_t)ctx->tune.conv_tilepx;
     for (uint32_t th = 1; th <= max_px && th <= g.H_out; ++th)
         for (uint32_t tw = 1; th * tw <= max_px && tw <= g.W_out; ++tw) {
             const uint64_t tiles = (uint64_t)so_ceil_div(g.H_out, th) * so_ceil_div(g.W_out, tw);
@@ -803,14 +803,13 @@ static so_status conv2d_dispatch(so_ctx *ctx, const so_conv_plan *plan, const fl
     // Batch entries per lane: as many as divide B and keep 16/8-byte alignment.
     const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY | (uintptr_t)dResid;
     int maxvec = 4;
-    if (const char *e = getenv("SPARSEOPS_CONV_VEC")) maxvec = atoi(e);
+    if (ctx->tune.conv_vec > 0) maxvec = ctx->tune.conv_vec;
     // The LDS-windowed kernel when the plan carries its layout and the batch splits into tiles of
     // 16, 8 or 4 (SPARSEOPS_CONV_WINDOW=1 forces it whenever possible, =0 forbids it: tuning and tests).
     const uint32_t lpp = window_lpp(B);
     if (plan->win.cc != 0 && lpp != 0 && (align & 15) == 0 && (uint64_t)plan->win.cc * g.H_in * g.W_in * B < (1ull << 31)) {
-        const char *force = getenv("SPARSEOPS_CONV_WINDOW");
-        const bool forced = force && force[0] == '1';
-        if (!(force && force[0] == '0')) {
+        const bool forced = ctx->tune.conv_window == 1;
+        if (ctx->tune.conv_window != 0) {
             bool done = false;
             const so_status s = lpp == 4 ? window_launch<4>(ctx, plan, dX, B, dBias, dResid, dY, act, forced, &done)
                               : lpp == 2 ? window_launch<2>(ctx, plan, dX, B, dBias, dResid, dY, act, forced, &done)

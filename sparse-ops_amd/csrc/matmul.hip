@@ -433,8 +433,7 @@ extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX
                  (size_t)ctx->max_lds_bytes >= so_tiled::kLdsBytes;
     if (tiled) {
         const uint64_t groups = (uint64_t)so_ceil_div(C, so_tiled::kSlabCols) * so_ceil_div(E->tiled.nquads, kTiledWaves);
-        const char *force = getenv("SPARSEOPS_MATMUL_TILED");
-        if (force) tiled = force[0] == '1';
+        if (ctx->tune.matmul_tiled >= 0) tiled = ctx->tune.matmul_tiled == 1;
         else tiled = 4 * groups >= 3 * (uint64_t)ctx->compute_units;
     }
     if (tiled) {
@@ -454,10 +453,7 @@ extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX
     int vec = 1;
     if (C % 256 == 0 && (align & 15) == 0) vec = 4;
     else if (C % 128 == 0 && (align & 7) == 0) vec = 2;
-    if (const char *e = getenv("SPARSEOPS_MATMUL_VEC")) {   // tuning override: narrower lanes only
-        const int v = atoi(e);
-        if ((v == 1 || v == 2) && v < vec) vec = v;
-    }
+    if ((ctx->tune.matmul_vec == 1 || ctx->tune.matmul_vec == 2) && ctx->tune.matmul_vec < vec) vec = ctx->tune.matmul_vec;   // narrower lanes only
     // Few waves in total (at most one per SIMD even with one column per lane): the
     // launch is latency-bound, so spread it over as many waves as possible and give
     // each wave 2 x 32 gathers in flight.

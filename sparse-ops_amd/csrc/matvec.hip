@@ -22,7 +22,6 @@
 #include "so_internal.h"
 
 #include <algorithm>
-#include <cstdlib>
 
 namespace {
 
@@ -291,12 +290,9 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
         // Lanes per row by the longest row (one pass of 16 G slots should cover it), but never so
         // few that compute units are left without rows.
         uint32_t G = E->max_nnz <= 128 ? 8u : E->max_nnz <= 256 ? 16u : E->max_nnz <= 512 ? 32u : 64u;
-        if (const char *e = getenv("SPARSEOPS_MATVEC_LANES")) {
-            const int v = atoi(e);
-            if (v == 8 || v == 16 || v == 32 || v == 64) G = (uint32_t)v;
-        } else {
+        if (ctx->tune.matvec_lanes) G = (uint32_t)ctx->tune.matvec_lanes;
+        else
             while (G < 64 && so_ceil_div(E->m, kWavesPerBlock * (64u / G)) < cus) G *= 2;
-        }
         // One resident workgroup per compute unit (the pipelined rows need the registers); each of
         // its 16 waves keeps two passes' loads in flight.
         const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, kWavesPerBlock * (64u / G)), cus));

@@ -35,6 +35,32 @@ extern "C" so_status so_device_count(int *n)
     return SO_OK;
 }
 
+static int env_int(const char *name, int unset)
+{
+    const char *e = getenv(name);
+    return (e && e[0]) ? atoi(e) : unset;
+}
+
+static void read_tuning(so_tuning &t)
+{
+    t = so_tuning();
+    t.matmul_tiled = env_int("SPARSEOPS_MATMUL_TILED", -1);
+    t.matmul_vec = env_int("SPARSEOPS_MATMUL_VEC", 0);
+    const int lanes = env_int("SPARSEOPS_MATVEC_LANES", 0);
+    t.matvec_lanes = (lanes == 8 || lanes == 16 || lanes == 32 || lanes == 64) ? lanes : 0;
+    t.conv_window = env_int("SPARSEOPS_CONV_WINDOW", -1);
+    t.conv_cpw = env_int("SPARSEOPS_CONV_CPW", 0);
+    t.conv_tilepx = env_int("SPARSEOPS_CONV_TILEPX", 0);
+    t.conv_vec = env_int("SPARSEOPS_CONV_VEC", 0);
+}
+
+extern "C" so_status so_tuning_reload(so_ctx *ctx)
+{
+    SO_REQUIRE(ctx != nullptr, "so_tuning_reload: ctx is null");
+    read_tuning(ctx->tune);
+    return SO_OK;
+}
+
 extern "C" so_status so_init(int device, so_ctx **out)
 {
     SO_REQUIRE(out != nullptr, "so_init: out is null");
@@ -52,6 +78,7 @@ extern "C" so_status so_init(int device, so_ctx **out)
     ctx->compute_units = prop.multiProcessorCount;
     ctx->max_lds_bytes = (int)prop.sharedMemPerBlock;
     ctx->name = prop.gcnArchName;
+    read_tuning(ctx->tune);
     hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev0);
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev1);

@@ -8,6 +8,18 @@
 
 #include "sparseops_hip.h"
 
+// Tuning overrides, read from the environment when the context is created (and again by
+// so_tuning_reload), never per launch.  0 / -1 = the library's own choice.
+struct so_tuning {
+    int matmul_tiled = -1;   // SPARSEOPS_MATMUL_TILED: 1 forces the LDS-staged kernel, 0 forbids it
+    int matmul_vec = 0;      // SPARSEOPS_MATMUL_VEC: 1 or 2 columns per lane at most
+    int matvec_lanes = 0;    // SPARSEOPS_MATVEC_LANES: 8, 16, 32 or 64 lanes per row
+    int conv_window = -1;    // SPARSEOPS_CONV_WINDOW: 1 forces the LDS-windowed kernel, 0 forbids it
+    int conv_cpw = 0;        // SPARSEOPS_CONV_CPW: most output channels per wave
+    int conv_tilepx = 0;     // SPARSEOPS_CONV_TILEPX: most output pixels per tile
+    int conv_vec = 0;        // SPARSEOPS_CONV_VEC: most batch entries per lane in the gather kernel
+};
+
 struct so_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -16,6 +28,7 @@ struct so_ctx {
     int max_lds_bytes = 0;   // largest LDS allocation one workgroup may ask for
     bool capturing = false;
     std::string name;
+    so_tuning tune;
 };
 
 // Rows of one length class for the binned matvec: `group` lanes cooperate on a row.

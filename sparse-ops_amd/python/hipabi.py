@@ -3,6 +3,7 @@
 This is the stub a maintainer of a Python caller would write; the tests and the
 benchmark drive the HIP kernels through it with device-resident operands.
 """
+import contextlib
 import ctypes as ct
 import os
 
@@ -17,7 +18,7 @@ LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS, LAYOUT_TILED = 1, 2, 4, 8
 
 # Every symbol include/sparseops_hip.h declares.
 SYMBOLS = (
-    "so_device_count so_init so_destroy so_last_error so_device_info so_malloc so_free so_h2d so_d2h "
+    "so_device_count so_init so_destroy so_last_error so_device_info so_tuning_reload so_malloc so_free so_h2d so_d2h "
     "so_d2d so_fill_zero so_sync so_timer_begin so_timer_end so_ellpack_upload so_ellpack_free "
     "so_ellpack_dims so_ellpack_download so_ellpack_decode so_ellpack_encode so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
     "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_graph_begin so_graph_end "
@@ -61,6 +62,7 @@ def load_library(path=None):
         "so_init": [ct.c_int, ct.POINTER(_vp)],
         "so_destroy": [_vp],
         "so_device_info": [_vp, ct.c_char_p, ct.c_size_t, ct.POINTER(ct.c_int)],
+        "so_tuning_reload": [_vp],
         "so_malloc": [_vp, ct.c_size_t, ct.POINTER(_vp)],
         "so_free": [_vp, _vp],
         "so_h2d": [_vp, _vp, _vp, ct.c_size_t],
@@ -193,6 +195,32 @@ class Context:
 
     def sync(self):
         self._ck(self.lib.so_sync(self.h))
+
+    def reload_tuning(self):
+        """Read the SPARSEOPS_* tuning overrides from the environment again (they are read once,
+        when the context is created)."""
+        self._ck(self.lib.so_tuning_reload(self.h))
+
+    @contextlib.contextmanager
+    def tuning(self, **overrides):
+        """with ctx.tuning(SPARSEOPS_MATMUL_TILED="1"): ...  -- set overrides (None unsets), reload,
+        and put everything back afterwards."""
+        saved = {k: os.environ.get(k) for k in overrides}
+        try:
+            for k, v in overrides.items():
+                if v is None:
+                    os.environ.pop(k, None)
+                else:
+                    os.environ[k] = str(v)
+            self.reload_tuning()
+            yield self
+        finally:
+            for k, v in saved.items():
+                if v is None:
+                    os.environ.pop(k, None)
+                else:
+                    os.environ[k] = v
+            self.reload_tuning()
 
     def timer_begin(self):
         self._ck(self.lib.so_timer_begin(self.h))

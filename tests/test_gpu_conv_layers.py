@@ -2,7 +2,6 @@
 the GPU against the oracle: bit-exact for everything whose arithmetic is fixed
 (conv with NONE/RELU, max, the ordered GAP sum, add, relu, transpose), 1e-6
 relative for the sigmoid/tanh library calls."""
-import os
 
 import numpy as np
 import pytest
@@ -20,14 +19,10 @@ def gpu_conv(ctx, E, g, X, B, bias, act="none", window=None, residual=None):
     False forbids it, None leaves the library's own choice."""
     dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
     plan = ctx.conv_plan(dE, g)
-    if window is not None:
-        os.environ["SPARSEOPS_CONV_WINDOW"] = "1" if window else "0"
-        if window:
-            assert ctx.conv_plan_window(plan) is not None and B % 4 == 0
-    try:
+    if window:
+        assert ctx.conv_plan_window(plan) is not None and B % 4 == 0
+    with ctx.tuning(SPARSEOPS_CONV_WINDOW=None if window is None else ("1" if window else "0")):
         return _gpu_conv(ctx, dE, plan, g, X, B, bias, act, residual)
-    finally:
-        os.environ.pop("SPARSEOPS_CONV_WINDOW", None)
 
 
 def _gpu_conv(ctx, dE, plan, g, X, B, bias, act, residual=None):

@@ -2,7 +2,6 @@
 oracle.  NONE/RELU epilogues must be bit-identical to the oracle (same rounding
 sequence: bias, then one FMA per stored nonzero in ascending slot order);
 SIGMOID/TANH use the device's expf/tanhf and must agree to 1e-6 relative."""
-import os
 
 import numpy as np
 import pytest
@@ -19,12 +18,9 @@ ACT_TOL = 1e-6
 
 def gpu_matmul(ctx, E, X, bias, act="none", layouts=hipabi.LAYOUT_ROW):
     # small test shapes would be routed to the row kernel: force the LDS-staged one
-    # whenever its layout is requested (library tuning override, read per call)
-    os.environ["SPARSEOPS_MATMUL_TILED"] = "1" if layouts & hipabi.LAYOUT_TILED else "0"
-    try:
+    # whenever its layout is requested (library tuning override)
+    with ctx.tuning(SPARSEOPS_MATMUL_TILED="1" if layouts & hipabi.LAYOUT_TILED else "0"):
         return _gpu_matmul(ctx, E, X, bias, act, layouts)
-    finally:
-        del os.environ["SPARSEOPS_MATMUL_TILED"]
 
 
 def _gpu_matmul(ctx, E, X, bias, act, layouts):

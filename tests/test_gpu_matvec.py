@@ -70,7 +70,7 @@ def test_matvec_every_row_written_once(ctx):
 
 @pytest.mark.parametrize("lanes", [8, 16, 32, 64])
 @pytest.mark.parametrize("m,n,kmax", [(3001, 1000, 203), (517, 4099, 700), (64, 300, 17), (70000, 256, 40)])
-def test_matvec_rows_lanes_per_row(ctx, monkeypatch, lanes, m, n, kmax):
+def test_matvec_rows_lanes_per_row(ctx, lanes, m, n, kmax):
     """The row kernel shares a row among 8, 16, 32 or 64 lanes (picked by the longest row and the
     row count; forced here): ragged rows including empty ones, odd r, rows longer than one pass."""
     rng = np.random.default_rng(lanes + m)
@@ -86,11 +86,10 @@ def test_matvec_rows_lanes_per_row(ctx, monkeypatch, lanes, m, n, kmax):
     y64 = b.astype(np.float64)
     for i in range(m):
         y64[i] += vals[i].astype(np.float64) @ x[cols[i]]
-    monkeypatch.setenv("SPARSEOPS_MATVEC_LANES", str(lanes))
-    y = gpu_matvec(ctx, E, x, b, layouts=hipabi.LAYOUT_ROW, which=(hipabi.LAYOUT_ROW,))[hipabi.LAYOUT_ROW]
+    with ctx.tuning(SPARSEOPS_MATVEC_LANES=lanes):
+        y = gpu_matvec(ctx, E, x, b, layouts=hipabi.LAYOUT_ROW, which=(hipabi.LAYOUT_ROW,))[hipabi.LAYOUT_ROW]
     assert np.isfinite(y).all()
     assert rel_err(y, y64) <= TOL
-    monkeypatch.delenv("SPARSEOPS_MATVEC_LANES")
     y_auto = gpu_matvec(ctx, E, x, b, layouts=hipabi.LAYOUT_ROW, which=(hipabi.LAYOUT_ROW,))[hipabi.LAYOUT_ROW]
     assert rel_err(y_auto, y64) <= TOL
 
