@@ -29,6 +29,7 @@ import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 VALU_FP32_PEAK_TF = 157.3    # MI355X vector fp32 (packed FMA); 78.6 with plain v_fma_f32
+LDS_OPERAND_PEAK_TF = 39.3   # 256 CUs x 128 B/clk of LDS reads x 2.4 GHz / 4 B per multiply-add x 2 flop
 # HBM-side bytes per launch of the headline kernel, from two rocprofv3 --pmc runs
 # (FETCH_SIZE, WRITE_SIZE) scaled by a plain copy of known size; see the pmc summary
 # under profiles/.  None until measured for the kernel that currently runs.
@@ -346,7 +347,14 @@ def main():
                      "row_kernel_us": round(ev_ms_row * 1e3, 2), "row_kernel_same_bits": row_bits_equal,
                      "valu_fp32_frac_of_157.3TF": round(flops / (ev_ms * 1e-3) / 1e12 / VALU_FP32_PEAK_TF, 4),
                      "valu_fp32_frac_of_78.6TF_unpacked": round(flops / (ev_ms * 1e-3) / 1e12 / (VALU_FP32_PEAK_TF / 2), 4),
-                     "binding_bound": "fp32 VALU / L1-L2 gather bandwidth (t_valu 10.9 us unpacked > t_hbm 2.7 us)"},
+                     # every multiply-add needs a 4-byte X operand from LDS/L1 (no reuse in registers):
+                     # bytes at that level, and the fraction of what LDS can deliver (128 B/clk/CU)
+                     "gather_bytes": 8 * E.total_nnz + 4 * E.total_nnz * C + 4 * E.m * C,
+                     "lds_operand_frac_of_39.3TF": round(flops / (ev_ms * 1e-3) / 1e12 / LDS_OPERAND_PEAK_TF, 4),
+                     "t_hbm_us": round(nbytes / (HBM_PEAK_GBS * 1e9) * 1e6, 2),
+                     "t_valu_us_unpacked": round(flops / (VALU_FP32_PEAK_TF / 2 * 1e12) * 1e6, 2),
+                     "t_bound_over_t": round(max(nbytes / (HBM_PEAK_GBS * 1e9), flops / (VALU_FP32_PEAK_TF / 2 * 1e12)) / (ev_ms * 1e-3), 4),
+                     "binding_bound": "operand delivery from LDS, then fp32 VALU issue (t_valu 10.9 us unpacked > t_hbm 2.7 us)"},
     }
     if args.calibrate_copy:
         # A plain copy of known size (act_kernel<NONE>: reads N floats, writes N floats)
