@@ -385,6 +385,18 @@ def main():
                                  "GBps": round(8 * n_cp / cp_ms / 1e6, 1), "hbm_frac": round(8 * n_cp / cp_ms / 1e6 / HBM_PEAK_GBS, 4)}
         src.free()
         dst.free()
+        # config 1 (1024x1024, C=64): a parity shape whose kernel is shorter than a launch; launches back to back
+        E1, X1, b1, _ = datagen.config1()
+        dE1 = ctx.upload_ellpack(E1.Wd, E1.idx, E1.nnz, E1.m, E1.n, E1.r, hipabi.LAYOUT_ROW)
+        dX1, dB1, dY1 = ctx.array(X1), ctx.array(b1), ctx.empty((E1.m, 64))
+        _, ms1 = time_launches(ctx, lambda: ctx.matmul(dE1, dX1, 64, dB1, dY1, "none"), max(100, args.steps), args.warmup)
+        extras["matmul_config1"] = {"workload": "ellpack_matmul 1024x1024 Bernoulli(0.1), C=64 (r=%d, nnz=%d), launches back to back"
+                                                % (E1.r, E1.total_nnz),
+                                    "us_per_launch": round(ms1 * 1e3, 2),
+                                    "nnz_gflops": round(2.0 * E1.total_nnz * 64 / ms1 / 1e6, 1)}
+        for a in (dX1, dB1, dY1):
+            a.free()
+        dE1.free()
         log("matvec 16384^2 uniform ...")
         extras["matvec_uniform"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 16384x16384, 95% Bernoulli",
                                                 datagen.config2a, hipabi.LAYOUT_ROW, hipabi.LAYOUT_ROW, k, args.warmup, not args.no_cpu)

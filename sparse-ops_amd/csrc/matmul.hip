@@ -423,6 +423,8 @@ extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX
     if (E->m == 0 || C == 0) return SO_OK;  // empty output: nothing to launch
     SO_REQUIRE(dY != nullptr, "so_matmul: Y is null");
     SO_REQUIRE(dX != nullptr || E->total_nnz == 0, "so_matmul: X is null");
+    // one workgroup per (4 rows, 64 columns) at most: the grid must fit 31 bits
+    SO_REQUIRE(((uint64_t)E->m / 4 + 8) * ((uint64_t)C / 64 + 1) < (1ull << 31), "so_matmul: %u x %u output is too large for one launch", E->m, C);
 
     const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY;
     // The LDS-staged kernel needs whole float4 column groups.  It takes one
