@@ -446,27 +446,24 @@ void window_launch_act(so_ctx *ctx, const so_conv_plan *plan, const WinArgs &a, 
 // The windowed kernels use more than the default 64 KB of dynamic LDS: raise the limit of every
 // instantiation once, at plan creation (never from so_conv2d, which may run under graph capture).
 template <int CPW, int LPP>
-hipError_t window_allow_lds(int bytes)
+hipError_t window_allow_lds(so_ctx *ctx)
 {
     hipError_t e = hipSuccess;
     const void *k[4] = {(const void *)conv2d_window_kernel<CPW, LPP, SO_ACT_NONE>, (const void *)conv2d_window_kernel<CPW, LPP, SO_ACT_RELU>,
                         (const void *)conv2d_window_kernel<CPW, LPP, SO_ACT_SIGMOID>, (const void *)conv2d_window_kernel<CPW, LPP, SO_ACT_TANH>};
     for (const void *f : k)
-        if (e == hipSuccess) e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e == hipSuccess) e = so_allow_big_lds(ctx, f);
     return e;
 }
 
 so_status window_configure(so_ctx *ctx)
 {
-    static bool configured = false;
-    if (configured) return SO_OK;
-    SO_HIP((window_allow_lds<8, 4>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<4, 4>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<2, 4>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<1, 4>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<8, 2>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<4, 2>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<2, 2>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<1, 2>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<8, 1>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<4, 1>(ctx->max_lds_bytes)));
-    SO_HIP((window_allow_lds<2, 1>(ctx->max_lds_bytes))); SO_HIP((window_allow_lds<1, 1>(ctx->max_lds_bytes)));
-    configured = true;
+    SO_HIP((window_allow_lds<8, 4>(ctx))); SO_HIP((window_allow_lds<4, 4>(ctx)));
+    SO_HIP((window_allow_lds<2, 4>(ctx))); SO_HIP((window_allow_lds<1, 4>(ctx)));
+    SO_HIP((window_allow_lds<8, 2>(ctx))); SO_HIP((window_allow_lds<4, 2>(ctx)));
+    SO_HIP((window_allow_lds<2, 2>(ctx))); SO_HIP((window_allow_lds<1, 2>(ctx)));
+    SO_HIP((window_allow_lds<8, 1>(ctx))); SO_HIP((window_allow_lds<4, 1>(ctx)));
+    SO_HIP((window_allow_lds<2, 1>(ctx))); SO_HIP((window_allow_lds<1, 1>(ctx)));
     return SO_OK;
 }
 

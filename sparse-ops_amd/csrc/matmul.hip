@@ -399,12 +399,7 @@ template <int ACT>
 so_status launch_tiled(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, const float *dBias, float *dY)
 {
     const so_tiled &T = E->tiled;
-    static thread_local bool configured = false;
-    if (!configured) {
-        SO_HIP(hipFuncSetAttribute((const void *)ellpack_matmul_tiled_kernel<ACT>,
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)so_tiled::kLdsBytes));
-        configured = true;
-    }
+    SO_HIP(so_allow_big_lds(ctx, (const void *)ellpack_matmul_tiled_kernel<ACT>));
     const uint32_t nslabs = so_ceil_div(C, so_tiled::kSlabCols);
     const uint32_t ngroups = so_ceil_div(T.nquads, kTiledWaves);
     const uint32_t blocks = (8 % nslabs == 0) ? so_ceil_div(ngroups, 8 / nslabs) * 8 : nslabs * ngroups;

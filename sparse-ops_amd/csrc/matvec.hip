@@ -244,25 +244,12 @@ void matvec_slot_kernel(const float *__restrict__ WdT, const uint32_t *__restric
 // LDS staging of x is worth its per-workgroup copy only when a workgroup then
 // serves many nonzeros from it; it needs n floats of LDS (set up once per kernel).
 template <typename K>
-bool use_lds(const so_ctx *ctx, K kernel, uint32_t n, uint64_t nnz_total, uint32_t blocks)
+bool use_lds(so_ctx *ctx, K kernel, uint32_t n, uint64_t nnz_total, uint32_t blocks)
 {
     const size_t lds = (size_t)n * sizeof(float);
     if (lds == 0 || lds > (size_t)ctx->max_lds_bytes) return false;
     if (nnz_total < (uint64_t)n * blocks) return false;   // fewer gathers than staged elements
-    if (lds > 48 * 1024) {
-        static thread_local const void *configured[8] = {};
-        const void *k = (const void *)kernel;
-        bool done = false;
-        for (const void *c : configured) done |= (c == k);
-        if (!done) {
-            if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, ctx->max_lds_bytes) != hipSuccess) {
-                (void)hipGetLastError();
-                return false;
-            }
-            for (const void *&c : configured)
-                if (!c) { c = k; break; }
-        }
-    }
+    if (lds > 48 * 1024 && so_allow_big_lds(ctx, (const void *)kernel) != hipSuccess) return false;
     return true;
 }
 

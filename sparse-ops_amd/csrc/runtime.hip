@@ -35,6 +35,16 @@ extern "C" so_status so_device_count(int *n)
     return SO_OK;
 }
 
+hipError_t so_allow_big_lds(so_ctx *ctx, const void *kernel)
+{
+    for (const void *k : ctx->big_lds_kernels)
+        if (k == kernel) return hipSuccess;
+    const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, ctx->max_lds_bytes);
+    if (e == hipSuccess) ctx->big_lds_kernels.push_back(kernel);
+    else (void)hipGetLastError();
+    return e;
+}
+
 static int env_int(const char *name, int unset)
 {
     const char *e = getenv(name);

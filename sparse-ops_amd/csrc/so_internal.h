@@ -29,6 +29,7 @@ struct so_ctx {
     bool capturing = false;
     std::string name;
     so_tuning tune;
+    std::vector<const void *> big_lds_kernels;   // kernels already allowed max_lds_bytes of dynamic LDS on this device
 };
 
 // Rows of one length class for the binned matvec: `group` lanes cooperate on a row.
@@ -81,6 +82,10 @@ struct so_graph {
 };
 
 void so_set_error(const char *fmt, ...);
+
+// Kernels that ask for more than 48 KB of dynamic LDS must be told so once per device: this does
+// it the first time `kernel` is seen on the context's device (hipSuccess when already done).
+hipError_t so_allow_big_lds(so_ctx *ctx, const void *kernel);
 
 #define SO_HIP(call)                                                              \
     do {                                                                          \
