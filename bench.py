@@ -404,6 +404,11 @@ def main():
         extras["matvec_zipf"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048",
                                              datagen.config2b, hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS, hipabi.LAYOUT_BINS,
                                              k, args.warmup, not args.no_cpu)
+        log("matvec 65536x16384 uniform ...")
+        # four times the rows of config 2a: what the same kernel streams once its fixed per-launch cost is amortised
+        extras["matvec_uniform_65536_rows"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 65536x16384, 95% Bernoulli",
+                                                           lambda: datagen.uniform_ellpack(48, 65536, 16384, 0.05),
+                                                           hipabi.LAYOUT_ROW, hipabi.LAYOUT_ROW, max(10, k // 4), 3, False)
         log("sparse MLP ...")
         extras["mlp"] = bench_mlp(k, args.warmup, with_cpu=not args.no_cpu)
         log("sparse CNN ...")

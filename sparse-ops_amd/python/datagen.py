@@ -86,6 +86,29 @@ def config2a(seed=43, m=16384, n=16384, keep=0.05):
     return E, x, bias
 
 
+def uniform_ellpack(seed, m, n, keep, chunk=4096):
+    """Bernoulli(keep) mask with N(0,1) values, built straight into ELLPACK arrays (for matrices
+    whose dense form would not fit).  A Bernoulli row is drawn through its gaps: the distances
+    between consecutive nonzeros are i.i.d. Geometric(keep), so the cost is O(nnz), not O(m n)."""
+    rng = np.random.default_rng(seed)
+    kmax = int(n * keep + 10 * np.sqrt(n * keep * (1 - keep)) + 16)
+    Wd = np.zeros((m, kmax), dtype=np.float32)
+    idx = np.zeros((m, kmax), dtype=np.uint32)
+    nnz = np.zeros(m, dtype=np.uint32)
+    for i0 in range(0, m, chunk):
+        rows = min(chunk, m - i0)
+        cols = np.cumsum(rng.geometric(keep, size=(rows, kmax)), axis=1, dtype=np.int64) - 1
+        live = cols < n
+        assert not live[:, -1].any(), "kmax too small for this draw"
+        nnz[i0:i0 + rows] = live.sum(axis=1)
+        idx[i0:i0 + rows] = np.where(live, cols, 0)
+        Wd[i0:i0 + rows] = np.where(live, rng.standard_normal((rows, kmax), dtype=np.float32), np.float32(0))
+    r = int(nnz.max()) if m else 0
+    x = rng.standard_normal(n, dtype=np.float32)
+    bias = rng.standard_normal(m, dtype=np.float32) * np.float32(0.1)
+    return EllpackHost(m, n, r, Wd[:, :r], idx[:, :r], nnz), x, bias
+
+
 def config2b(seed=44, m=16384, n=16384, s=1.2, cap=2048):
     """matvec, skewed: per-row nnz = min(Zipf(s), cap) (clipped, so a fifth of the
     rows sit at the cap and r = cap), columns uniform without replacement, ascending."""
