@@ -116,3 +116,19 @@ def test_datagen_encoder_matches(oracle):
     W[17] = 0
     E, Eo = datagen.encode_dense(W), oracle.encode(W)
     assert E.r == Eo.r and np.array_equal(E.Wd, Eo.Wd) and np.array_equal(E.idx, Eo.idx) and np.array_equal(E.nnz, Eo.nnz)
+
+
+def test_datagen_gap_generator_is_a_valid_encoding(oracle):
+    """uniform_ellpack builds ELLPACK arrays without the dense matrix: they must be exactly what
+    the encoder makes of the matrix they describe, with the requested density."""
+    import datagen
+    E, x, b = datagen.uniform_ellpack(5, 300, 2000, 0.05)
+    assert x.shape == (2000,) and b.shape == (300,)
+    W = np.zeros((300, 2000), np.float32)
+    for i in range(300):
+        c = E.idx[i, :E.nnz[i]]
+        assert (np.diff(c.astype(np.int64)) > 0).all() and (c < 2000).all()
+        W[i, c] = E.Wd[i, :E.nnz[i]]
+    Eo = oracle.encode(W)
+    assert E.r == Eo.r and np.array_equal(E.Wd, Eo.Wd) and np.array_equal(E.idx, Eo.idx) and np.array_equal(E.nnz, Eo.nnz)
+    assert abs(E.total_nnz / (300 * 2000) - 0.05) < 0.005
