@@ -134,7 +134,7 @@ int main(int argc, char **argv)
 {
     if (argc < 2 || (std::strcmp(argv[1], "matmul") && std::strcmp(argv[1], "matvec"))) {
         std::fprintf(stderr, "usage: %s matmul|matvec --M <rows> --N <cols> [--C <cols of X>] --sparsity <p> --runs <r> "
-                             "--seed <s> --irregular <0|1>\n", argv[0]);
+                             "--seed <s> --irregular <0|1> [--device <id>]\n", argv[0]);
         return 1;
     }
     const bool matmul = !std::strcmp(argv[1], "matmul");
@@ -143,6 +143,7 @@ int main(int argc, char **argv)
     double sparsity = 0.9;
     uint64_t seed = 42;
     bool irregular = false;
+    int device = 0;
     for (int i = 2; i < argc; ++i) {
         const std::string a = argv[i];
         if (i + 1 >= argc) { std::fprintf(stderr, "incomplete arg: %s\n", a.c_str()); return 1; }
@@ -153,6 +154,7 @@ int main(int argc, char **argv)
         else if (a == "--runs") runs = std::stoi(argv[++i]);
         else if (a == "--seed") seed = std::stoull(argv[++i]);
         else if (a == "--irregular") irregular = std::stoi(argv[++i]) != 0;
+        else if (a == "--device") device = std::stoi(argv[++i]);
         else { std::fprintf(stderr, "unknown arg: %s\n", a.c_str()); return 1; }
     }
     if (!matmul) C = 1;
@@ -171,7 +173,8 @@ int main(int argc, char **argv)
     std::printf("nnz %zu, ELLPACK r %u (padding %.2fx)\n\n", nnz_total, h.r, nnz_total ? double(M) * h.r / nnz_total : 0.0);
 
     so_ctx *ctx = nullptr;
-    SOCK(so_init(0, &ctx));
+    HIPCK(hipSetDevice(device));
+    SOCK(so_init(device, &ctx));
     hipStream_t stream = nullptr;                     // vendor libraries run on the null stream
     float *dX = to_device(X), *dW = to_device(h.W), *dval = to_device(h.values);
     int *drow = to_device(h.row_ptr), *dcol = to_device(h.col_ind);
