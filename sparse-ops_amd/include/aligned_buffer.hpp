@@ -1,34 +1,57 @@
-// 64-byte aligned, move-only float buffer.  Same surface as the reference's
-// AlignedBuffer (include/aligned_buffer.hpp:8-30: members `ptr` and `size`,
-// throws std::bad_alloc); the allocation is left uninitialised.
+// Float storage on a 64-byte boundary with single ownership.  Source-compatible with the
+// reference's AlignedBuffer (include/aligned_buffer.hpp:8-30): public `ptr` and `size`,
+// construction from an element count, std::bad_alloc on failure, movable but not copyable.
+// Contents start uninitialised.
 #pragma once
 
 #include <cstddef>
 #include <cstdlib>
 #include <new>
-#include <utility>
 
 struct AlignedBuffer {
-    float *ptr = nullptr;
-    std::size_t size = 0;
+    static constexpr std::size_t kAlign = 64;
 
-    AlignedBuffer() = default;
-    explicit AlignedBuffer(std::size_t count) : size(count)
+    float *ptr;
+    std::size_t size;
+
+    AlignedBuffer() noexcept : ptr(nullptr), size(0) {}
+
+    explicit AlignedBuffer(std::size_t count) : ptr(nullptr), size(count)
     {
-        const std::size_t bytes = ((count * sizeof(float) + 63) / 64) * 64;
-        ptr = static_cast<float *>(std::aligned_alloc(64, bytes ? bytes : 64));
-        if (!ptr) throw std::bad_alloc();
+        // posix_memalign accepts any size, zero included (a distinct pointer that free() takes)
+        void *mem = nullptr;
+        if (posix_memalign(&mem, kAlign, count ? count * sizeof(float) : kAlign) != 0) throw std::bad_alloc();
+        ptr = static_cast<float *>(mem);
     }
-    ~AlignedBuffer() { std::free(ptr); }
+
+    AlignedBuffer(AlignedBuffer &&from) noexcept : AlignedBuffer() { take(from); }
+
+    AlignedBuffer &operator=(AlignedBuffer &&from) noexcept
+    {
+        if (this != &from) {
+            drop();
+            take(from);
+        }
+        return *this;
+    }
 
     AlignedBuffer(const AlignedBuffer &) = delete;
     AlignedBuffer &operator=(const AlignedBuffer &) = delete;
-    AlignedBuffer(AlignedBuffer &&other) noexcept
-        : ptr(std::exchange(other.ptr, nullptr)), size(std::exchange(other.size, 0)) {}
-    AlignedBuffer &operator=(AlignedBuffer &&other) noexcept
+
+    ~AlignedBuffer() { drop(); }
+
+  private:
+    void drop() noexcept
     {
-        std::swap(ptr, other.ptr);
-        std::swap(size, other.size);
-        return *this;
+        std::free(ptr);
+        ptr = nullptr;
+        size = 0;
+    }
+    void take(AlignedBuffer &from) noexcept
+    {
+        ptr = from.ptr;
+        size = from.size;
+        from.ptr = nullptr;
+        from.size = 0;
     }
 };

@@ -1,9 +1,17 @@
-// ELLPACK container and host encoder.  Drop-in for the reference's
-// include/ellpack_encoder.hpp:6-32: same struct members, same free functions.
-// The one addition is `device`, an opaque handle to the matrix's copy in HBM,
-// created on first use by ellpack_matmul / ellpack_matvec and shared by copies.
+// ELLPACK container and host encoder: source-compatible with the reference's
+// include/ellpack_encoder.hpp:6-32 (a caller may construct an Ellpack, read and write its
+// members, and call the two free functions exactly as there).
+//
+// Layout: row i owns slots [i*r, (i+1)*r) of Wd and idx; its first nnz[i] slots hold the row's
+// nonzero values and their column numbers in ascending column order, the rest hold 0.0f / 0.
+// r is the largest nnz[i].  Xt (the reference's gather scratch for matvec) is allocated so that
+// code touching it still works, and never read by this library.
+//
+// Addition: `device`, the matrix's copy in GPU memory.  ellpack_matmul / ellpack_matvec create it
+// on first use; copies of the struct made afterwards share it.
 #pragma once
 
+#include <cstddef>
 #include <cstdint>
 #include <memory>
 #include <vector>
@@ -13,25 +21,30 @@
 namespace sparseops { struct EllpackMirror; }
 
 struct Ellpack {
-    uint32_t m;  ///< rows
-    uint32_t n;  ///< columns of the dense matrix
-    uint32_t r;  ///< slots per row = max nonzeros of any row
+    uint32_t m;                  // rows
+    uint32_t n;                  // columns of the dense matrix
+    uint32_t r;                  // slots per row
+    AlignedBuffer Wd;            // m*r values
+    std::vector<uint32_t> idx;   // m*r column numbers
+    AlignedBuffer Xt;            // m*r floats, unused (see above)
+    std::vector<uint32_t> nnz;   // m counts of stored nonzeros
+    mutable std::shared_ptr<sparseops::EllpackMirror> device;
 
-    AlignedBuffer Wd;           ///< m*r values, row-major, zero padded
-    std::vector<uint32_t> idx;  ///< m*r column indices, zero padded
-    AlignedBuffer Xt;           ///< m*r floats; host scratch kept for source compatibility, unused here
-    std::vector<uint32_t> nnz;  ///< m stored-nonzero counts
+    Ellpack(uint32_t rows, uint32_t cols, uint32_t slots_per_row)
+        : m(rows), n(cols), r(slots_per_row), Wd(slot_count(rows, slots_per_row)),
+          idx(slot_count(rows, slots_per_row), 0u), Xt(slot_count(rows, slots_per_row)), nnz(rows, 0u)
+    {
+    }
 
-    mutable std::shared_ptr<sparseops::EllpackMirror> device;  ///< HBM copy, lazily created
+    std::size_t slots() const { return slot_count(m, r); }
 
-    Ellpack(uint32_t m_, uint32_t n_, uint32_t r_)
-        : m(m_), n(n_), r(r_), Wd(std::size_t(m_) * r_), idx(std::size_t(m_) * r_),
-          Xt(std::size_t(m_) * r_), nnz(m_) {}
+  private:
+    static std::size_t slot_count(uint32_t rows, uint32_t per_row) { return std::size_t(rows) * per_row; }
 };
 
-/// Encode a dense row-major m x n matrix (reference: src/ellpack_encoder.cpp:6-44).
+// Dense row-major m x n -> ELLPACK (reference: src/ellpack_encoder.cpp:6-44).
 Ellpack convert_to_ellpack(const float *W, uint32_t m, uint32_t n);
 
-/// Decode into a dense m x n matrix; W_out holds m*n floats
-/// (reference: src/ellpack_encoder.cpp:46-60).
+// ELLPACK -> dense row-major m x n; W_out has room for m*n floats and is overwritten entirely
+// (reference: src/ellpack_encoder.cpp:46-60).
 void decode_from_ellpack(const Ellpack &E, float *W_out);

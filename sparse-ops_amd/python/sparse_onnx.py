@@ -1,8 +1,11 @@
-"""Pure-Python ONNX runner on top of the ELLPACK kernels: the reference's
-OnnxSparseModel (python/sparse_onnx.py:6-53) without the `onnx` package -- the graph
-is read by the bundled wire-format reader.  A 1-D input runs through matvec, a 2-D
-(n, C) input through matmul, activations in numpy, exactly as the reference does;
-as there, Gemm/MatMul weights are encoded as stored (out x in for a PyTorch Gemm)."""
+"""Pure-Python ONNX runner on top of the ELLPACK kernels.
+
+Same class, constructor and `run` as the reference's OnnxSparseModel
+(python/sparse_onnx.py:6-53), without the `onnx` package: the file is read by the bundled
+wire-format reader.  Behaviour kept from the reference: Gemm/MatMul weights are encoded as they
+are stored (out x in for a PyTorch Gemm), a Gemm's third input is its bias, a 1-D input goes
+through matvec and a 2-D (n, C) input through matmul, Relu/Sigmoid/Tanh run in numpy, any other
+operator raises NotImplementedError when the model is built."""
 import numpy as np
 
 try:
@@ -13,32 +16,41 @@ except ImportError:          # imported as top-level modules (sys.path points at
     from cpp_backend import encode, matmul, matvec
 
 
+def _product_step(E, bias):
+    def step(v):
+        return (matvec if v.ndim == 1 else matmul)(E, v, bias)
+    return step
+
+
+_ELEMENTWISE = {
+    "Relu": lambda v: np.maximum(v, 0),
+    "Sigmoid": lambda v: (1 / (1 + np.exp(-v))).astype(np.float32),
+    "Tanh": np.tanh,
+}
+
+
 class OnnxSparseModel:
     def __init__(self, onnx_path: str):
         with open(onnx_path, "rb") as f:
             graph = onnx_wire.read_model(f.read())
-        self._initializers = {k: v.astype(np.float32) for k, v in graph["initializers"].items()}
-        self.layers = []
+        self._initializers = {name: arr.astype(np.float32) for name, arr in graph["initializers"].items()}
+        self.layers = []      # (name, Ellpack or None, bias or None), one per node: the reference's plan, for inspection
+        self._steps = []      # what run() calls, in order
         for node in graph["nodes"]:
-            op = node["op_type"]
-            if op in ("Gemm", "MatMul"):
-                W = self._initializers[node["input"][1]]
-                b = self._initializers[node["input"][2]] if op == "Gemm" and len(node["input"]) > 2 else None
-                self.layers.append(("matmul", encode(W), b))
-            elif op in ("Relu", "Sigmoid", "Tanh"):
-                self.layers.append((op.lower(), None, None))
+            kind, operands = node["op_type"], node["input"]
+            if kind in ("Gemm", "MatMul"):
+                E = encode(self._initializers[operands[1]])
+                bias = self._initializers[operands[2]] if kind == "Gemm" and len(operands) > 2 else None
+                self.layers.append(("matmul", E, bias))
+                self._steps.append(_product_step(E, bias))
+            elif kind in _ELEMENTWISE:
+                self.layers.append((kind.lower(), None, None))
+                self._steps.append(_ELEMENTWISE[kind])
             else:
-                raise NotImplementedError("Unsupported op %s" % op)
+                raise NotImplementedError("Unsupported op %s" % kind)
 
     def run(self, x: np.ndarray) -> np.ndarray:
-        v = x.astype(np.float32)
-        for op, E, b in self.layers:
-            if op == "matmul":
-                v = matvec(E, v, b) if v.ndim == 1 else matmul(E, v, b)
-            elif op == "relu":
-                v = np.maximum(v, 0)
-            elif op == "sigmoid":
-                v = (1 / (1 + np.exp(-v))).astype(np.float32)
-            elif op == "tanh":
-                v = np.tanh(v)
+        v = np.asarray(x, dtype=np.float32)
+        for step in self._steps:
+            v = step(v)
         return v
