@@ -1,0 +1,112 @@
+// A C++ caller written against the reference's headers only (ellpack_encoder.hpp,
+// ellpack_matmul.hpp, ellpack_matvec.hpp, sparse_onnx.hpp): host pointers in, host pointers out,
+// as benchmark-mkl/matmul/bench_matmul.cpp:98 and benchmark-mkl/matvec/bench_matvec.cpp:100 of the
+// reference call them.  Checks every result against plain loops and exits non-zero on a mismatch.
+//
+//   dropin_consumer                      kernels only
+//   dropin_consumer model.onnx in.bin expected.bin B     + SparseOnnxModel::run, bit for bit
+#include "ellpack_encoder.hpp"
+#include "ellpack_matmul.hpp"
+#include "ellpack_matvec.hpp"
+#include "sparse_onnx.hpp"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <random>
+#include <vector>
+
+static int failures = 0;
+static void check(bool ok, const char *what)
+{
+    std::printf("%s %s\n", ok ? "ok  " : "FAIL", what);
+    if (!ok) ++failures;
+}
+
+static std::vector<float> read_floats(const char *path)
+{
+    std::ifstream f(path, std::ios::binary | std::ios::ate);
+    std::vector<float> v(f ? (size_t)f.tellg() / sizeof(float) : 0);
+    f.seekg(0);
+    f.read(reinterpret_cast<char *>(v.data()), (std::streamsize)(v.size() * sizeof(float)));
+    return v;
+}
+
+int main(int argc, char **argv)
+{
+    const uint32_t m = 300, n = 200, C = 72;
+    std::mt19937 rng(7);
+    std::normal_distribution<float> gauss;
+    std::uniform_real_distribution<float> coin(0.0f, 1.0f);
+    std::vector<float> W(size_t(m) * n), X(size_t(n) * C), bias(m), x(n);
+    for (auto &v : W) v = coin(rng) < 0.85f ? 0.0f : gauss(rng);
+    for (auto &v : X) v = gauss(rng);
+    for (auto &v : bias) v = gauss(rng);
+    for (auto &v : x) v = gauss(rng);
+    std::fill(W.begin() + 5 * n, W.begin() + 6 * n, 0.0f);          // an empty row
+
+    Ellpack E = convert_to_ellpack(W.data(), m, n);
+    std::vector<float> back(size_t(m) * n, -1.0f);
+    decode_from_ellpack(E, back.data());
+    check(std::memcmp(back.data(), W.data(), back.size() * sizeof(float)) == 0, "decode(encode(W)) == W");
+    check(E.m == m && E.n == n && E.nnz[5] == 0 && E.Wd.size == size_t(m) * E.r && E.idx.size() == size_t(m) * E.r,
+          "Ellpack members");
+
+    // the reference's rounding sequence: bias, then one fused multiply-add per stored slot in order
+    std::vector<float> want(size_t(m) * C), got(size_t(m) * C, NAN);
+    for (uint32_t i = 0; i < m; ++i)
+        for (uint32_t c = 0; c < C; ++c) {
+            float acc = bias[i];
+            for (uint32_t k = 0; k < E.nnz[i]; ++k) acc = std::fmaf(E.Wd.ptr[size_t(i) * E.r + k], X[size_t(E.idx[size_t(i) * E.r + k]) * C + c], acc);
+            want[size_t(i) * C + c] = acc;
+        }
+    ellpack_matmul(E, X.data(), C, bias.data(), got.data());
+    check(std::memcmp(got.data(), want.data(), got.size() * sizeof(float)) == 0, "ellpack_matmul bit-exact");
+
+    std::fill(got.begin(), got.end(), NAN);
+    ellpack_matmul_fused<false, true>(E, X.data(), C, bias.data(), got.data());
+    bool relu_ok = true;
+    for (size_t i = 0; i < got.size(); ++i) relu_ok &= got[i] == (want[i] > 0.0f ? want[i] : 0.0f);
+    check(relu_ok, "ellpack_matmul_fused<false, true> (fused ReLU)");
+
+    std::fill(got.begin(), got.end(), NAN);
+    ellpack_matmul(E, X.data(), C, nullptr, got.data());
+    bool nobias_ok = true;
+    for (uint32_t i = 0; i < m && nobias_ok; ++i) {
+        float acc = 0.0f;
+        for (uint32_t k = 0; k < E.nnz[i]; ++k) acc = std::fmaf(E.Wd.ptr[size_t(i) * E.r + k], X[size_t(E.idx[size_t(i) * E.r + k]) * C], acc);
+        nobias_ok = got[size_t(i) * C] == acc;
+    }
+    check(nobias_ok, "ellpack_matmul with bias == nullptr");
+
+    std::vector<float> y(m, NAN);
+    ellpack_matvec(E, x.data(), bias.data(), y.data());
+    double worst = 0.0, scale = 0.0;
+    for (uint32_t i = 0; i < m; ++i) {
+        double acc = bias[i];
+        for (uint32_t j = 0; j < n; ++j) acc += double(W[size_t(i) * n + j]) * x[j];
+        worst = std::max(worst, std::fabs(acc - y[i]));
+        scale = std::max(scale, std::fabs(acc));
+    }
+    check(worst <= 1e-5 * scale, "ellpack_matvec within 1e-5 of the fp64 product");
+
+    if (argc == 5) {
+        const uint32_t B = (uint32_t)std::atoi(argv[4]);
+        const std::vector<float> in = read_floats(argv[2]), expected = read_floats(argv[3]);
+        SparseOnnxModel model(argv[1]);
+        const std::vector<size_t> shape = model.output_shape();
+        size_t out_count = 1;
+        for (size_t d : shape) out_count *= d;
+        check(!shape.empty() && shape[0] == B && out_count == expected.size(), "SparseOnnxModel::output_shape");
+        std::vector<float> out(expected.size(), NAN);
+        model.run(in.data(), B, out.data());
+        check(std::memcmp(out.data(), expected.data(), out.size() * sizeof(float)) == 0, "SparseOnnxModel::run bit-exact");
+        model.resize_buffers(B);
+        std::fill(out.begin(), out.end(), NAN);
+        model.run(in.data(), B, out.data());
+        check(std::memcmp(out.data(), expected.data(), out.size() * sizeof(float)) == 0, "run after resize_buffers");
+    }
+    std::printf("%d failure(s)\n", failures);
+    return failures ? 1 : 0;
+}

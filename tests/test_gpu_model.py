@@ -298,3 +298,27 @@ def test_resnet18_full_size_batch_independence(backend, oracle, tmp_path):
     assert np.array_equal(model.run(X), Y)                       # back to 32 after the resizes
     from graph_oracle import run_graph
     assert np.array_equal(run_graph(oracle, payload, X[:1]), Y[:1])
+
+
+def test_cpp_caller_of_the_reference_headers(oracle, tmp_path):
+    """tests/cpp/dropin_consumer.cpp is a C++ program written against the reference's headers
+    (host pointers, as its benchmark drivers call the kernels): encoder round trip, ellpack_matmul
+    and the fused-ReLU instantiation bit for bit, ellpack_matvec within 1e-5, and
+    SparseOnnxModel::run / resize_buffers on a Gemm+ReLU chain bit for bit against the oracle."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "dropin_consumer")
+    assert os.path.exists(exe), "tests/cpp/dropin_consumer is not built (run __graft_entry__.build())"
+    rng = np.random.default_rng(12)
+    dims, B = (40, 96, 70, 13), 20
+    Ws = [datagen.magnitude_prune(rng.standard_normal((o, i)).astype(np.float32), .75) for i, o in zip(dims[:-1], dims[1:])]
+    bs = [rng.standard_normal(o).astype(np.float32) for o in dims[1:]]
+    acts = ["Relu", "Relu", None]
+    path = ow.save(str(tmp_path / "mlp.onnx"), ow.mlp_model(Ws, acts, B, bs, True))
+    X = rng.standard_normal((B, 40)).astype(np.float32)
+    Yo = oracle_mlp(oracle, Ws, acts, X, bs)                       # (B, 13)
+    np.ascontiguousarray(X.T).tofile(str(tmp_path / "in.bin"))     # [features x B], the C++ contract
+    np.ascontiguousarray(Yo.T).tofile(str(tmp_path / "expected.bin"))
+    r = subprocess.run([exe, path, str(tmp_path / "in.bin"), str(tmp_path / "expected.bin"), str(B)],
+                       capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count("ok  ") == 9 and "FAIL" not in r.stdout
