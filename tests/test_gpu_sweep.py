@@ -1,0 +1,100 @@
+"""Seeded random sweep over shapes the hand-picked cases do not list: convolution geometry
+(kernel, stride, dilation, padding, ragged tiles, any batch), matmul and matvec shapes, every
+kernel variant the library can take for them, against the oracle (bit-exact for matmul and
+convolution, 1e-5 relative for matvec)."""
+import numpy as np
+import pytest
+
+from conftest import as_oracle
+
+import datagen
+import hipabi
+
+pytestmark = pytest.mark.gpu
+
+
+def _sparse(rng, m, n, sp):
+    W = rng.standard_normal((m, n)).astype(np.float32)
+    W[rng.random((m, n)) < sp] = 0
+    return W
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_convolutions(ctx, oracle, seed):
+    from oracle import conv_geom as ocg
+    rng = np.random.default_rng(seed)
+    for it in range(40):
+        Cin, Cout = int(rng.integers(1, 40)), int(rng.integers(1, 40))
+        k = (int(rng.integers(1, 6)), int(rng.integers(1, 6)))
+        s = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        d = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        p = (int(rng.integers(0, 4)), int(rng.integers(0, 4)))
+        H = int(rng.integers(d[0] * (k[0] - 1) + 1, 30))
+        Wi = int(rng.integers(d[1] * (k[1] - 1) + 1, 30))
+        B = int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16, 20, 32, 48]))
+        Wc = _sparse(rng, Cout, Cin * k[0] * k[1], float(rng.choice([0.0, 0.3, 0.6, 0.9, 0.98])))
+        if Cout > 2:
+            Wc[int(rng.integers(0, Cout))] = 0
+        X = rng.standard_normal((Cin, H, Wi, B)).astype(np.float32)
+        b = rng.standard_normal(Cout).astype(np.float32) if rng.random() < 0.7 else None
+        act = str(rng.choice(["none", "relu"]))
+        case = "seed %d case %d: Cin=%d Cout=%d k=%s s=%s d=%s p=%s H=%d W=%d B=%d act=%s" % (seed, it, Cin, Cout, k, s, d, p, H, Wi, B, act)
+        E = datagen.encode_dense(Wc)
+        g, og = hipabi.conv_geom(Cin, Cout, k[0], k[1], H, Wi, s, p, d), ocg(Cin, Cout, k[0], k[1], H, Wi, s, p, d)
+        want = oracle.conv2d_pf(as_oracle(E), og, X, B, b, act)
+        dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+        plan = ctx.conv_plan(dE, g)
+        dX, dY = ctx.array(X), ctx.empty((Cout, g.H_out, g.W_out, B))
+        dB = ctx.array(b) if b is not None else None
+        for window in (None, "0", "1"):
+            if window == "1" and (ctx.conv_plan_window(plan) is None or B % 4):
+                continue
+            with ctx.tuning(SPARSEOPS_CONV_WINDOW=window):
+                dY.upload(np.full((Cout, g.H_out, g.W_out, B), np.nan, np.float32))
+                ctx.conv2d(plan, dX, B, dB, dY, act)
+                assert np.array_equal(dY.download(), want), "%s window=%s" % (case, window)
+        ctx.conv_plan_free(plan)
+        dE.free()
+        for a in (dX, dY, dB):
+            if a is not None:
+                a.free()
+
+
+@pytest.mark.parametrize("seed", [21, 22, 23])
+def test_random_products(ctx, oracle, seed):
+    rng = np.random.default_rng(seed)
+    every = hipabi.LAYOUT_ROW | hipabi.LAYOUT_SLOT | hipabi.LAYOUT_BINS | hipabi.LAYOUT_TILED
+    for it in range(40):
+        m, n = int(rng.integers(1, 400)), int(rng.integers(1, 700))
+        C = int(rng.choice([1, 3, 4, 16, 20, 64, 68, 100, 128, 256, 260]))
+        W = _sparse(rng, m, n, float(rng.choice([0.0, 0.5, 0.9, 0.99])))
+        if m > 3:
+            W[2] = 0
+        E = datagen.encode_dense(W)
+        X = rng.standard_normal((n, C)).astype(np.float32)
+        b = rng.standard_normal(m).astype(np.float32) if rng.random() < 0.7 else None
+        act = str(rng.choice(["none", "relu"]))
+        case = "seed %d case %d: m=%d n=%d C=%d act=%s" % (seed, it, m, n, C, act)
+        want = oracle.matmul(as_oracle(E), X, b, act)
+        dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, every)
+        dX, dY = ctx.array(X), ctx.empty((m, C))
+        dB = ctx.array(b) if b is not None else None
+        for tiled in ("0", "1"):
+            with ctx.tuning(SPARSEOPS_MATMUL_TILED=tiled):
+                dY.upload(np.full((m, C), np.nan, np.float32))
+                ctx.matmul(dE, dX, C, dB, dY, act)
+                assert np.array_equal(dY.download(), want), "%s tiled=%s" % (case, tiled)
+        x = rng.standard_normal(n).astype(np.float32)
+        dx, dy = ctx.array(x), ctx.empty((m,))
+        y64 = W.astype(np.float64) @ x + (b if b is not None else 0)
+        for layout in (hipabi.LAYOUT_ROW, hipabi.LAYOUT_SLOT, hipabi.LAYOUT_BINS, 0):
+            for lanes in ((None, 8, 16, 32, 64) if layout == hipabi.LAYOUT_ROW else (None,)):
+                with ctx.tuning(SPARSEOPS_MATVEC_LANES=lanes):
+                    dy.upload(np.full(m, np.nan, np.float32))
+                    ctx.matvec(dE, dx, dB, dy, layout)
+                    err = np.abs(dy.download() - y64).max() / max(np.abs(y64).max(), 1e-30)
+                assert err <= 1e-5, "%s matvec layout=%d lanes=%s err=%g" % (case, layout, lanes, err)
+        dE.free()
+        for a in (dX, dY, dB, dx, dy):
+            if a is not None:
+                a.free()
