@@ -98,3 +98,35 @@ def test_random_products(ctx, oracle, seed):
         for a in (dX, dY, dB, dx, dy):
             if a is not None:
                 a.free()
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_random_pool_add_transpose(ctx, oracle, seed):
+    rng = np.random.default_rng(seed)
+    for it in range(40):
+        C, H, Wi = int(rng.integers(1, 20)), int(rng.integers(1, 25)), int(rng.integers(1, 25))
+        B = int(rng.choice([1, 2, 3, 4, 6, 8, 16, 20, 32]))
+        k = (int(rng.integers(1, min(H, 4) + 1)), int(rng.integers(1, min(Wi, 4) + 1)))
+        s = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        pad = (int(rng.integers(0, k[0])), int(rng.integers(0, k[1])))       # a window always meets the image
+        X = rng.standard_normal((C, H, Wi, B)).astype(np.float32)
+        case = "seed %d case %d: C=%d H=%d W=%d B=%d k=%s s=%s pad=%s" % (seed, it, C, H, Wi, B, k, s, pad)
+        want = oracle.maxpool_pf(X, C, H, Wi, B, k, s, pad)
+        dX, dY = ctx.array(X), ctx.empty(want.shape)
+        ctx.maxpool(C, H, Wi, k, s, pad, dX, B, dY)
+        assert np.array_equal(dY.download(), want), case
+        dG = ctx.empty((C, B))
+        ctx.gap(C, H, Wi, dX, B, dG)
+        assert np.array_equal(dG.download(), oracle.gap_pf(X, C, H, Wi, B)), case
+        R = rng.standard_normal(X.shape).astype(np.float32)
+        dR, dS = ctx.array(R), ctx.empty(X.shape)
+        ctx.add(dX, dR, X.size, dS)
+        assert np.array_equal(dS.download(), oracle.add(X, R)), case
+        ctx.act("relu", dS, X.size, dS)
+        assert np.array_equal(dS.download(), oracle.act(oracle.add(X, R), "relu")), case
+        rows, cols = C * H, Wi * B
+        dT = ctx.empty((cols, rows))
+        ctx.transpose(dX, rows, cols, dT)
+        assert np.array_equal(dT.download(), X.reshape(rows, cols).T), case
+        for a in (dX, dY, dG, dR, dS, dT):
+            a.free()
