@@ -130,3 +130,107 @@ def test_random_pool_add_transpose(ctx, oracle, seed):
         assert np.array_equal(dT.download(), X.reshape(rows, cols).T), case
         for a in (dX, dY, dG, dR, dS, dT):
             a.free()
+
+
+def _random_cnn(rng, B):
+    """A random graph of the operators the loader supports with exact arithmetic: Conv (bias or not,
+    random kernel/stride/padding) + optional Relu, MaxPool, residual blocks (Conv-Relu-Conv + skip,
+    the skip either the block's input or a 1x1 projection, Add, optional Relu), then
+    GlobalAveragePool or Flatten and a Gemm head."""
+    import onnx_wire as ow
+    nodes, inits = [], []
+    C, H, W = int(rng.integers(1, 5)), int(rng.integers(9, 21)), int(rng.integers(9, 21))
+    shape_in = (B, C, H, W)
+    cur, uid = "input", [0]
+
+    def name(prefix):
+        uid[0] += 1
+        return "%s%d" % (prefix, uid[0])
+
+    def conv(src, cin, cout, k, s, p, relu):
+        nonlocal H, W
+        w = rng.standard_normal((cout, cin, k, k)).astype(np.float32) * np.float32(0.3)
+        w[rng.random(w.shape) < 0.6] = 0
+        wn, out = name("w"), name("conv")
+        inits.append((wn, w))
+        ins = [src, wn]
+        if rng.random() < 0.6:
+            bn = name("b")
+            inits.append((bn, rng.standard_normal(cout).astype(np.float32)))
+            ins.append(bn)
+        nodes.append(ow.node("Conv", ins, [out], kernel_shape=[k, k], strides=[s, s], pads=[p, p, p, p], dilations=[1, 1], group=1))
+        Ho, Wo = (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1
+        if relu:
+            r = name("relu")
+            nodes.append(ow.node("Relu", [out], [r]))
+            out = r
+        return out, Ho, Wo
+
+    for _ in range(int(rng.integers(1, 4))):
+        kind = rng.choice(["conv", "block", "pool"])
+        if kind == "conv":
+            cout, k = int(rng.integers(2, 12)), int(rng.choice([1, 3, 5]))
+            s, p = int(rng.integers(1, 3)), int(rng.integers(0, k // 2 + 1))
+            if H + 2 * p < k or W + 2 * p < k:
+                continue
+            cur, H, W = conv(cur, C, cout, k, s, p, rng.random() < 0.7)
+            C = cout
+        elif kind == "block":
+            cout, s = int(rng.integers(2, 12)), int(rng.integers(1, 3))
+            a, Ha, Wa = conv(cur, C, cout, 3, s, 1, True)
+            H0, W0 = H, W
+            H, W = Ha, Wa
+            b2, H, W = conv(a, cout, cout, 3, 1, 1, False)
+            if s == 1 and cout == C and rng.random() < 0.5:
+                skip = cur
+            else:
+                H, W = H0, W0
+                skip, H, W = conv(cur, C, cout, 1, s, 0, False)
+            out = name("add")
+            nodes.append(ow.node("Add", [b2, skip] if rng.random() < 0.5 else [skip, b2], [out]))
+            if rng.random() < 0.7:
+                r = name("relu")
+                nodes.append(ow.node("Relu", [out], [r]))
+                out = r
+            cur, C = out, cout
+        elif H >= 3 and W >= 3:
+            k, s = int(rng.integers(2, 4)), int(rng.integers(1, 3))
+            p = int(rng.integers(0, k // 2 + 1))
+            out = name("pool")
+            nodes.append(ow.node("MaxPool", [cur], [out], kernel_shape=[k, k], strides=[s, s], pads=[p, p, p, p]))
+            cur, H, W = out, (H + 2 * p - k) // s + 1, (W + 2 * p - k) // s + 1
+    if rng.random() < 0.5:
+        nodes.append(ow.node("GlobalAveragePool", [cur], ["gap"]))
+        nodes.append(ow.node("Flatten", ["gap"], ["flat"], axis=1))
+        feats = C
+    else:
+        nodes.append(ow.node("Flatten", [cur], ["flat"], axis=1))
+        feats = C * H * W
+    classes = int(rng.integers(1, 9))
+    fw = rng.standard_normal((classes, feats)).astype(np.float32)
+    fw[rng.random(fw.shape) < 0.5] = 0
+    inits += [("fcw", fw), ("fcb", rng.standard_normal(classes).astype(np.float32))]
+    nodes.append(ow.node("Gemm", ["flat", "fcw", "fcb"], ["output"], alpha=1.0, beta=1.0, transB=1))
+    return ow.model(nodes, [("input", shape_in)], [("output", (B, classes))], inits), shape_in
+
+
+@pytest.mark.parametrize("seed", [41, 42, 43, 44])
+def test_random_cnn_graphs(backend, oracle, tmp_path, seed):
+    """Whole models: loader (shape inference, fusions), planner, device chain and launch graph on
+    random graphs, bit for bit against the oracle's layer-by-layer execution of the same file."""
+    import onnx_wire as ow
+    from graph_oracle import run_graph
+    rng = np.random.default_rng(seed)
+    for it in range(10):
+        B = int(rng.choice([1, 2, 3, 4, 8, 16]))
+        payload, shape_in = _random_cnn(rng, B)
+        path = ow.save(str(tmp_path / ("g%d.onnx" % it)), payload)
+        model = backend.SparseOnnxModel(path)
+        X = rng.standard_normal(shape_in).astype(np.float32)
+        want = run_graph(oracle, payload, X)
+        got = model.run(X)
+        assert got.shape == want.shape and np.array_equal(got, want), "seed %d graph %d: %s" % (seed, it, model.describe())
+        assert np.array_equal(model.run(np.asfortranarray(X)), want)
+        B2 = int(rng.choice([1, 4, 5]))
+        X2 = rng.standard_normal((B2,) + tuple(shape_in[1:])).astype(np.float32)
+        assert np.array_equal(model.run(X2), run_graph(oracle, payload, X2)), "seed %d graph %d at batch %d" % (seed, it, B2)
