@@ -207,6 +207,12 @@ so_status so_act(so_ctx *ctx, int act, const float *dX, size_t len, float *dY);
  * array to the kernels' [F x B] layout and back (the reference's Python tests
  * do this on the host with Fortran-order arrays, tests/full_test.py:77-88). */
 so_status so_transpose(so_ctx *ctx, const float *dSrc, uint32_t rows, uint32_t cols, float *dDst);
+/* Copy a [rows x cols] matrix between buffers whose rows start src_stride / dst_stride floats
+ * apart; with zero_fill the rest of every destination row (cols .. dst_stride) is set to zero.
+ * No counterpart in the reference: the model runtime uses it to carry a batch that is not a
+ * multiple of four inside buffers that are (what the convolution kernels' batch tiles need). */
+so_status so_copy_rows(so_ctx *ctx, const float *dSrc, size_t src_stride, uint32_t rows, uint32_t cols,
+                       float *dDst, size_t dst_stride, int zero_fill);
 
 /* ---- launch graphs -------------------------------------------------------
  * Record every launch made on the context between begin and end into one

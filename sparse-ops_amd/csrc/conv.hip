@@ -36,6 +36,7 @@ struct so_conv_window {
     uint32_t TH = 0, TW = 0, IH = 0, IW = 0, cc = 0, nch = 0, tiles_x = 0, tiles_y = 0;
     uint32_t groups = 0;          // ceil(Cout / cpw)
     int cpw = 0;                  // output channels per wave
+    uint32_t lpp = 0;             // lanes per pixel (batch tile / 4) the chunk size was chosen for: 4, 2 or 1
     int2 *d_stream = nullptr;     // all groups' streams, followed by one padding quad
     uint32_t *d_gbase = nullptr;  // [groups]: first quad (4 entries) of the group's stream
     uint32_t *d_quads = nullptr;  // [groups * nch * cpw]: quads of (group, chunk, channel in group)
@@ -492,6 +493,8 @@ so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, 
     a.buf_f4 = (w.cc + 1) * w.IH * w.IW * LPP;
     a.nbuf = w.nch > 1 ? 2u : 1u;
     const size_t lds = (size_t)a.nbuf * a.buf_f4 * 16;
+    // a layout whose chunks were sized for a smaller batch tile than this batch's does not fit
+    if (LPP > w.lpp && (lds > (size_t)ctx->max_lds_bytes || a.win_f4 > (uint32_t)kWinMaxPerThread * kWinThreads)) return SO_OK;
     const dim3 grid(w.tiles_x * w.tiles_y, so_ceil_div(w.groups, a.cg), B / (4 * LPP));
     const uint64_t wgs = (uint64_t)grid.x * grid.y * grid.z;
     // Even a grid that covers an eighth of the chip beats the gather kernel on long rows (measured on the
@@ -592,10 +595,14 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     w.tiles_x = so_ceil_div(g.W_out, w.TW);
     if ((uint64_t)w.IH * w.IW > 4096) return SO_OK;
     // Channel chunk: two windows (plus their zero planes) fit LDS, one window fits the copy loop.
-    const uint64_t px_bytes = kWinBT * 4, lds_budget = (uint64_t)ctx->max_lds_bytes;
+    // Both depend on the batch tile (16, 8 or 4 entries): a smaller tile lets a chunk hold more
+    // channels, i.e. fewer chunks, fewer barriers and longer runs -- what small batches, whose
+    // launches are bound by latency, need.  A layout sized for a batch tile also serves smaller ones.
+    w.lpp = window_lpp(batch) ? window_lpp(batch) : kWinLPP;
+    const uint64_t px_bytes = w.lpp * 16, lds_budget = (uint64_t)ctx->max_lds_bytes;
     uint32_t cc = g.Cin;
     while (cc > 0 && ((cc < g.Cin ? 2ull : 1ull) * (cc + 1) * w.IH * w.IW * px_bytes > lds_budget ||
-                      (uint64_t)cc * w.IH * w.IW * kWinLPP > (uint64_t)kWinMaxPerThread * kWinThreads))
+                      (uint64_t)cc * w.IH * w.IW * w.lpp > (uint64_t)kWinMaxPerThread * kWinThreads))
         --cc;
     if (cc == 0) return SO_OK;
     w.nch = so_ceil_div(g.Cin, cc);
@@ -761,9 +768,11 @@ extern "C" so_status so_conv_plan_tune(so_ctx *ctx, so_conv_plan *plan, uint32_t
     const uint32_t batch = std::max(4u, B / 4u * 4u);
     if (batch == plan->tuned_batch || plan->win.cc == 0) return SO_OK;
     const so_ellpack *E = plan->E;
-    // Rebuild only if the batch changes the choice of channels per wave.
+    // Rebuild only if the batch changes the batch tile the chunks are sized for or the choice of
+    // channels per wave.
     const double run = (double)E->total_nnz / (double)plan->g.Cout / plan->win.nch;
-    if (choose_cpw(ctx, plan->win, plan->g.Cout, run, batch) == plan->win.cpw) {
+    const uint32_t lpp = window_lpp(batch) ? window_lpp(batch) : kWinLPP;
+    if (lpp == plan->win.lpp && choose_cpw(ctx, plan->win, plan->g.Cout, run, batch) == plan->win.cpw) {
         plan->tuned_batch = batch;
         return SO_OK;
     }

@@ -202,6 +202,32 @@ extern "C" so_status so_act(so_ctx *ctx, int act, const float *dX, size_t len, f
     return SO_OK;
 }
 
+// dst row i = src row i's first `cols` values, then zeros up to dst_stride (src_stride, dst_stride in floats).
+__global__ __launch_bounds__(kBlock)
+void copy_rows_kernel(const float *__restrict__ src, size_t src_stride, uint32_t cols, float *__restrict__ dst,
+                      size_t dst_stride, uint32_t dst_cols, size_t total)
+{
+    for (size_t e = (size_t)blockIdx.x * kBlock + threadIdx.x; e < total; e += (size_t)gridDim.x * kBlock) {
+        const size_t row = e / dst_cols;
+        const uint32_t c = (uint32_t)(e % dst_cols);
+        dst[row * dst_stride + c] = c < cols ? src[row * src_stride + c] : 0.0f;
+    }
+}
+
+extern "C" so_status so_copy_rows(so_ctx *ctx, const float *dSrc, size_t src_stride, uint32_t rows, uint32_t cols,
+                                  float *dDst, size_t dst_stride, int zero_fill)
+{
+    SO_REQUIRE(ctx != nullptr, "so_copy_rows: ctx is null");
+    if (rows == 0 || cols == 0) return SO_OK;
+    SO_REQUIRE(dSrc && dDst, "so_copy_rows: null tensor");
+    SO_REQUIRE(src_stride >= cols && dst_stride >= cols, "so_copy_rows: a stride is shorter than a row");
+    const uint32_t dst_cols = zero_fill ? (uint32_t)std::min<size_t>(dst_stride, 0xffffffffu) : cols;
+    const size_t total = (size_t)rows * dst_cols;
+    copy_rows_kernel<<<blocks_for(ctx, total), kBlock, 0, ctx->stream>>>(dSrc, src_stride, cols, dDst, dst_stride, dst_cols, total);
+    SO_LAUNCH_CHECK();
+    return SO_OK;
+}
+
 extern "C" so_status so_transpose(so_ctx *ctx, const float *dSrc, uint32_t rows, uint32_t cols, float *dDst)
 {
     SO_REQUIRE(ctx != nullptr, "so_transpose: ctx is null");

@@ -21,7 +21,7 @@ SYMBOLS = (
     "so_device_count so_init so_destroy so_last_error so_device_info so_tuning_reload so_malloc so_free so_h2d so_d2h "
     "so_d2d so_fill_zero so_sync so_timer_begin so_timer_end so_ellpack_upload so_ellpack_free "
     "so_ellpack_dims so_ellpack_download so_ellpack_decode so_ellpack_encode so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
-    "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_graph_begin so_graph_end "
+    "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_copy_rows so_graph_begin so_graph_end "
     "so_graph_launch so_graph_free").split()
 
 _vp = ct.c_void_p
@@ -92,6 +92,7 @@ def load_library(path=None):
         "so_add": [_vp, _vp, _vp, ct.c_size_t, _vp],
         "so_act": [_vp, ct.c_int, _vp, ct.c_size_t, _vp],
         "so_transpose": [_vp, _vp, _u32, _u32, _vp],
+        "so_copy_rows": [_vp, _vp, ct.c_size_t, _u32, _u32, _vp, ct.c_size_t, ct.c_int],
         "so_graph_begin": [_vp],
         "so_graph_end": [_vp, ct.POINTER(_vp)],
         "so_graph_launch": [_vp, _vp],
@@ -293,6 +294,9 @@ class Context:
 
     def transpose(self, dSrc, rows, cols, dDst):
         self._ck(self.lib.so_transpose(self.h, dSrc.ptr, rows, cols, dDst.ptr))
+
+    def copy_rows(self, dSrc, src_stride, rows, cols, dDst, dst_stride, zero_fill=False):
+        self._ck(self.lib.so_copy_rows(self.h, dSrc.ptr, src_stride, rows, cols, dDst.ptr, dst_stride, int(zero_fill)))
 
     def fill_zero(self, dA):
         self._ck(self.lib.so_fill_zero(self.h, dA.ptr, dA.nbytes))

@@ -56,11 +56,15 @@ struct SparseOnnxModel::Impl {
     std::vector<int> output_dims;  // shape of the graph output, batch first
     int input_slot = -1, output_slot = -1;
     std::size_t in_features = 0, out_features = 0;
-    uint32_t batch = 0;
+    uint32_t batch = 0;            // samples per call, as the caller sees it
+    uint32_t pbatch = 0;           // samples per row of every arena tensor: batch rounded up to a multiple of four when
+                                   // the model has convolutions (their LDS-windowed kernel works on batch tiles of 4+)
+    bool has_conv = false;
 
     sparseops::DeviceBuffer bias_pool;   // all biases, contiguous
     sparseops::DeviceBuffer arena;       // all activation slots
-    sparseops::DeviceBuffer stage_in, stage_out;  // batch-major staging for run_batch_major
+    sparseops::DeviceBuffer stage_in, stage_out;  // staging for the caller's layouts (batch-major, or unpadded rows)
+    sparseops::DeviceBuffer stage_mid;            // [features x batch] between a transpose and the padded arena rows
     so_graph *graph = nullptr;           // recorded layer chain (arena -> arena)
     bool use_graph = true;
 
@@ -68,4 +72,7 @@ struct SparseOnnxModel::Impl {
     float *slot_ptr(int s) const { return arena.f32() + slots[s].offset; }
     void enqueue_layers(const float *in, float *out) const;  // in/out override the arena slots when non-null
     void launch_chain() const;                               // graph replay or eager
+    bool padded() const { return pbatch != batch; }
+    void rows_in(const float *d_rows) const;                 // [in_features x batch] -> the input slot (rows padded with zeros)
+    void rows_out(float *d_rows) const;                      // the output slot -> [out_features x batch]
 };

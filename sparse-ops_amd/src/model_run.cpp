@@ -5,6 +5,7 @@
 // with an unchanged batch size allocates nothing.
 #include "sparse_onnx.hpp"
 
+#include <algorithm>
 #include <stdexcept>
 
 #include "model_impl.hpp"
@@ -18,18 +19,27 @@ void SparseOnnxModel::resize_buffers(uint32_t batch)
     so_ctx *ctx = context();
     std::lock_guard<std::mutex> lock(context_mutex());
     if (M.graph) { so_graph_free(ctx, M.graph); M.graph = nullptr; }
+    M.has_conv = false;
+    for (const LayerPlan &L : M.layers) M.has_conv |= L.conv != nullptr;
+    // A batch that is not a multiple of four would push every convolution onto the slower
+    // gather kernel: carry it in rows of the next multiple of four instead (the extra columns are
+    // zeros on input and are never copied out; batch entries do not interact).
+    const uint32_t pbatch = (M.has_conv && batch % 4 != 0) ? (batch + 3u) / 4u * 4u : batch;
     // Slot offsets for this batch, 256-byte aligned.
     std::size_t total = 0;
+    std::size_t widest = std::max(M.in_features, M.out_features);
     for (Slot &s : M.slots) {
         s.offset = total;
-        total += (s.features * batch + 63) / 64 * 64;
+        total += (s.features * pbatch + 63) / 64 * 64;
     }
     M.arena.reserve(total * sizeof(float));
     M.stage_in.reserve(M.in_features * batch * sizeof(float));
     M.stage_out.reserve(M.out_features * batch * sizeof(float));
+    if (pbatch != batch) M.stage_mid.reserve(widest * batch * sizeof(float));
     M.batch = batch;
+    M.pbatch = pbatch;
     for (const LayerPlan &L : M.layers)
-        if (L.conv) check(so_conv_plan_tune(ctx, L.conv, batch), "so_conv_plan_tune");
+        if (L.conv) check(so_conv_plan_tune(ctx, L.conv, pbatch), "so_conv_plan_tune");
     if (M.use_graph && !M.layers.empty()) {
         check(so_graph_begin(ctx), "so_graph_begin");
         try {
@@ -47,7 +57,7 @@ void SparseOnnxModel::resize_buffers(uint32_t batch)
 void SparseOnnxModel::Impl::enqueue_layers(const float *in, float *out) const
 {
     so_ctx *ctx = context();
-    const uint32_t B = batch;
+    const uint32_t B = pbatch;
     auto src = [&](int s) -> const float * { return (in && s == input_slot) ? in : slot_ptr(s); };
     auto dst = [&](int s) -> float * { return (out && s == output_slot) ? out : slot_ptr(s); };
     for (const LayerPlan &L : layers) {
@@ -84,15 +94,33 @@ void SparseOnnxModel::Impl::launch_chain() const
     else enqueue_layers(nullptr, nullptr);
 }
 
+void SparseOnnxModel::Impl::rows_in(const float *d_rows) const
+{
+    check(so_copy_rows(context(), d_rows, batch, uint32_t(in_features), batch, slot_ptr(input_slot), pbatch, 1), "so_copy_rows(input)");
+}
+
+void SparseOnnxModel::Impl::rows_out(float *d_rows) const
+{
+    check(so_copy_rows(context(), slot_ptr(output_slot), pbatch, uint32_t(out_features), batch, d_rows, batch, 0), "so_copy_rows(output)");
+}
+
 void SparseOnnxModel::run(const float *input, uint32_t B, float *output) const
 {
     Impl &M = *impl_;
     if (B != M.batch) const_cast<SparseOnnxModel *>(this)->resize_buffers(B);
     so_ctx *ctx = context();
     std::lock_guard<std::mutex> lock(context_mutex());
-    check(so_h2d(ctx, M.slot_ptr(M.input_slot), input, M.in_features * B * sizeof(float)), "so_h2d(input)");
+    if (!M.padded()) {
+        check(so_h2d(ctx, M.slot_ptr(M.input_slot), input, M.in_features * B * sizeof(float)), "so_h2d(input)");
+        M.launch_chain();
+        check(so_d2h(ctx, output, M.slot_ptr(M.output_slot), M.out_features * B * sizeof(float)), "so_d2h(output)");
+        return;
+    }
+    check(so_h2d(ctx, M.stage_in.get(), input, M.in_features * B * sizeof(float)), "so_h2d(input)");
+    M.rows_in(M.stage_in.f32());
     M.launch_chain();
-    check(so_d2h(ctx, output, M.slot_ptr(M.output_slot), M.out_features * B * sizeof(float)), "so_d2h(output)");
+    M.rows_out(M.stage_out.f32());
+    check(so_d2h(ctx, output, M.stage_out.get(), M.out_features * B * sizeof(float)), "so_d2h(output)");
 }
 
 void SparseOnnxModel::run_batch_major(const float *input, uint32_t B, float *output) const
@@ -102,9 +130,17 @@ void SparseOnnxModel::run_batch_major(const float *input, uint32_t B, float *out
     so_ctx *ctx = context();
     std::lock_guard<std::mutex> lock(context_mutex());
     check(so_h2d(ctx, M.stage_in.get(), input, M.in_features * B * sizeof(float)), "so_h2d(input)");
-    check(so_transpose(ctx, M.stage_in.f32(), B, uint32_t(M.in_features), M.slot_ptr(M.input_slot)), "so_transpose(input)");
-    M.launch_chain();
-    check(so_transpose(ctx, M.slot_ptr(M.output_slot), uint32_t(M.out_features), B, M.stage_out.f32()), "so_transpose(output)");
+    if (!M.padded()) {
+        check(so_transpose(ctx, M.stage_in.f32(), B, uint32_t(M.in_features), M.slot_ptr(M.input_slot)), "so_transpose(input)");
+        M.launch_chain();
+        check(so_transpose(ctx, M.slot_ptr(M.output_slot), uint32_t(M.out_features), B, M.stage_out.f32()), "so_transpose(output)");
+    } else {
+        check(so_transpose(ctx, M.stage_in.f32(), B, uint32_t(M.in_features), M.stage_mid.f32()), "so_transpose(input)");
+        M.rows_in(M.stage_mid.f32());
+        M.launch_chain();
+        M.rows_out(M.stage_mid.f32());
+        check(so_transpose(ctx, M.stage_mid.f32(), uint32_t(M.out_features), B, M.stage_out.f32()), "so_transpose(output)");
+    }
     check(so_d2h(ctx, output, M.stage_out.get(), M.out_features * B * sizeof(float)), "so_d2h(output)");
 }
 
@@ -116,6 +152,12 @@ void SparseOnnxModel::run_device(const float *dInput, uint32_t B, float *dOutput
     std::lock_guard<std::mutex> lock(context_mutex());
     if (M.layers.empty()) {
         check(so_d2d(context(), dOutput, dInput, M.in_features * B * sizeof(float)), "so_d2d");
+        return;
+    }
+    if (M.padded()) {
+        M.rows_in(dInput);
+        M.launch_chain();
+        M.rows_out(dOutput);
         return;
     }
     M.enqueue_layers(dInput, dOutput);

@@ -128,7 +128,16 @@ def test_random_pool_add_transpose(ctx, oracle, seed):
         dT = ctx.empty((cols, rows))
         ctx.transpose(dX, rows, cols, dT)
         assert np.array_equal(dT.download(), X.reshape(rows, cols).T), case
-        for a in (dX, dY, dG, dR, dS, dT):
+        # rows of `cols` floats into rows `stride` apart, the tail of every row zeroed, and back
+        stride = cols + int(rng.integers(0, 5))
+        dP = ctx.array(np.full((rows, stride), np.nan, np.float32))
+        ctx.copy_rows(dX, cols, rows, cols, dP, stride, zero_fill=True)
+        P = dP.download()
+        assert np.array_equal(P[:, :cols], X.reshape(rows, cols)) and not P[:, cols:].any(), case
+        dQ = ctx.array(np.full((rows, cols), np.nan, np.float32))
+        ctx.copy_rows(dP, stride, rows, cols, dQ, cols)
+        assert np.array_equal(dQ.download(), X.reshape(rows, cols)), case
+        for a in (dX, dY, dG, dR, dS, dT, dP, dQ):
             a.free()
 
 
