@@ -308,7 +308,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path shards over the dense-column axis "
-                 "with no exchange; see DESIGN.md); run with --gpus 1")
+                 "with no exchange: every GPU would take B/N of the batch against its own copy of the weights); run with --gpus 1")
 
     import datagen
     import hipabi
