@@ -289,11 +289,18 @@ def bench_cnn(steps, warmup, with_cpu=True):
         model = sb.SparseOnnxModel(ow.save(os.path.join(d, "r18.onnx"), payload))
     dev_ms = model.time_device(steps, warmup)
     flops = model.nnz_flops_per_sample() * 32
-    return {"workload": "ResNet-18-shaped conv stack (no BN), 80% sparse, B=32, 3x224x224, implicit im2col",
-            "cpu_baseline": cpu_baseline_cnn(payload, model) if with_cpu else None,
-            "layers": len(model.describe()), "ms_per_batch_device_resident": round(dev_ms, 3),
-            "samples_per_s_device_resident": round(32 / (dev_ms * 1e-3), 1),
-            "nnz_gflop_per_batch": round(flops / 1e9, 2), "nnz_gflops": round(flops / (dev_ms * 1e-3) / 1e9, 1)}
+    out = {"workload": "ResNet-18-shaped conv stack (no BN), 80% sparse, B=32, 3x224x224, implicit im2col",
+           "cpu_baseline": cpu_baseline_cnn(payload, model) if with_cpu else None,
+           "layers": len(model.describe()), "ms_per_batch_device_resident": round(dev_ms, 3),
+           "samples_per_s_device_resident": round(32 / (dev_ms * 1e-3), 1),
+           "nnz_gflop_per_batch": round(flops / 1e9, 2), "nnz_gflops": round(flops / (dev_ms * 1e-3) / 1e9, 1)}
+    # the same model at serving-sized batches (latency-bound): resize_buffers re-tunes the convolution plans
+    small = {}
+    for b in (1, 8):
+        model.resize_buffers(b)
+        small[str(b)] = round(model.time_device(steps, warmup), 3)
+    out["ms_per_batch_by_batch_size"] = small
+    return out
 
 
 def main():
