@@ -33,7 +33,7 @@ LDS_OPERAND_PEAK_TF = 39.3   # 256 CUs x 128 B/clk of LDS reads x 2.4 GHz / 4 B 
 # HBM-side bytes per launch of the headline kernel, from two rocprofv3 --pmc runs
 # (FETCH_SIZE, WRITE_SIZE) scaled by a plain copy of known size; see the pmc summary
 # under profiles/.  None until measured for the kernel that currently runs.
-MEASURED_TRAFFIC_BYTES = 91_300_000   # ellpack_matmul_tiled_kernel: 87.1 MB fetched + 4.19 MB written
+MEASURED_TRAFFIC_BYTES = 57_500_000   # ellpack_matmul_tiled_kernel: 53.3 MB fetched + 4.19 MB written
 # the same counters for the two matvec kernels (profiles/bench_all_kernels__pmc_hbm_bytes.txt)
 MEASURED_MATVEC_TRAFFIC = {"ellpack_matvec 16384x16384, 95% Bernoulli": 112_300_000,
                            "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048": 69_800_000}

@@ -287,16 +287,20 @@ void ellpack_matmul_tiled_kernel(const so_tile_entry *__restrict__ entries, cons
                                  const uint32_t *__restrict__ quad_rows, uint32_t nquads, uint32_t ntiles,
                                  uint32_t n, const float *__restrict__ X, uint32_t C,
                                  const float *__restrict__ bias, float *__restrict__ Y,
-                                 uint32_t nslabs, uint32_t ngroups)
+                                 uint32_t nslabs, uint32_t ngroups, bool group_major)
 {
     constexpr uint32_t KT = so_tiled::kTileRows, ROWB = so_tiled::kSlabCols * 4, TILE = so_tiled::kTileBytes;
     extern __shared__ __attribute__((aligned(16))) char lds[];
-    // Workgroup id -> (column slab, group of 16 quads); an XCD (id % 8) keeps to one
-    // slab when the slab count divides 8, so its L2 holds a single slab of X.
+    // Workgroup id -> (column slab, group of 16 quads).  Workgroup ids go round the 8 XCDs, each
+    // with its own L2.  group_major: an XCD takes whole groups, the slabs of a group one after the
+    // other, so the group's entries come from HBM once and from that L2 for the other slabs
+    // (chosen when all of X fits an L2).  Otherwise an XCD keeps to one slab when the slab count
+    // divides 8, so that its L2 has to hold a single slab of X.
     uint32_t slab, grp;
     {
         const uint32_t xcd = blockIdx.x & 7u, q = blockIdx.x >> 3;
-        if (8 % nslabs == 0) { slab = xcd % nslabs; grp = xcd / nslabs + (8 / nslabs) * q; }
+        if (group_major) { slab = q % nslabs; grp = (q / nslabs) * 8u + xcd; }
+        else if (8 % nslabs == 0) { slab = xcd % nslabs; grp = xcd / nslabs + (8 / nslabs) * q; }
         else { slab = blockIdx.x % nslabs; grp = blockIdx.x / nslabs; }
         if (grp >= ngroups) return;
     }
@@ -402,9 +406,12 @@ so_status launch_tiled(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32
     SO_HIP(so_allow_big_lds(ctx, (const void *)ellpack_matmul_tiled_kernel<ACT>));
     const uint32_t nslabs = so_ceil_div(C, so_tiled::kSlabCols);
     const uint32_t ngroups = so_ceil_div(T.nquads, kTiledWaves);
-    const uint32_t blocks = (8 % nslabs == 0) ? so_ceil_div(ngroups, 8 / nslabs) * 8 : nslabs * ngroups;
+    // all of X inside one XCD's L2 (4 MB): share a group's entries between its slabs instead of a slab between groups
+    const bool grpmajor = (uint64_t)E->n * C * sizeof(float) <= (4ull << 20);
+    const uint32_t blocks = grpmajor ? so_ceil_div(ngroups, 8) * 8 * nslabs
+                                     : (8 % nslabs == 0) ? so_ceil_div(ngroups, 8 / nslabs) * 8 : nslabs * ngroups;
     ellpack_matmul_tiled_kernel<ACT><<<blocks, kTiledWaves * 64, so_tiled::kLdsBytes, ctx->stream>>>(
-        T.d_entries, T.d_info, T.d_rows, T.nquads, T.ntiles, E->n, dX, C, dBias, dY, nslabs, ngroups);
+        T.d_entries, T.d_info, T.d_rows, T.nquads, T.ntiles, E->n, dX, C, dBias, dY, nslabs, ngroups, grpmajor);
     return SO_OK;
 }
 
