@@ -127,6 +127,19 @@ def test_matmul_lds_tiled_layout(ctx, oracle, m, n, C, sp, act):
             assert np.array_equal(Y, Yo)
 
 
+@pytest.mark.parametrize("m,n,C", [(300, 2100, 512), (260, 2100, 640), (520, 4200, 256), (130, 1100, 1024)])
+def test_matmul_lds_tiled_x_larger_than_an_l2(ctx, oracle, m, n, C):
+    """X above 4 MiB: the kernel deals column slabs (not whole row groups) to the XCDs,
+    with a slab count that divides 8 (C = 256, 512), does not (640), or exceeds it (1024)."""
+    assert n * C * 4 > 4 << 20
+    rng = np.random.default_rng(m + n + C)
+    W = sparse_matrix(rng, m, n, .9)
+    X = rng.standard_normal((n, C)).astype(np.float32)
+    b = rng.standard_normal(m).astype(np.float32)
+    E = datagen.encode_dense(W)
+    assert np.array_equal(gpu_matmul(ctx, E, X, b, "relu", TILED), oracle.matmul(as_oracle(E), X, b, "relu"))
+
+
 def test_matmul_lds_tiled_reference_vectors_and_config3(ctx, oracle, golden):
     E = datagen.encode_dense(golden["enc_W"])
     b = golden["mm_bias"]
