@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ELLPACK compute path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--spinup-ms T] [--no-extras] [--no-cpu]
 
 Headline workload ("step" = one ellpack_matmul launch over the whole dense block):
 the large FC configuration, W 4096 x 4096 fp32 N(0, 0.02) with per-row top-10 %
@@ -12,6 +12,9 @@ VALU fraction, and the same configuration timed on the host cores with the
 reference's own kernel (`oracle/_ref`, kind "reference") or, where that cannot run,
 the plain-C restatement (kind "port").  `extras` holds the other configurations:
 matvec 16384 x 16384 (uniform and Zipf-skewed rows) and the sparse MLP's samples/s.
+Every kernel timed on its own is first launched untimed for --spinup-ms (150 ms) so that the
+GPU's clocks have settled, then for the W warm-up steps, then timed for exactly K steps (the
+two models' chains are timed after their warm-up passes only: they gain nothing from it).
 """
 import argparse
 import json
@@ -49,8 +52,23 @@ def alg_bytes(nnz, m, n, C):
     return 8 * nnz + 4 * m + 4 * m + 4 * n * C + 4 * m * C
 
 
+SPINUP_MS = 150.0   # --spinup-ms
+
+
+def spin_up(ctx, fn):
+    """Untimed launches of `fn` for SPINUP_MS of wall time: after an idle spell (an upload, host
+    work) the GPU needs some 100 ms of continuous load before its clocks settle, and launches
+    timed before that read up to 14 % slow.  Comes before the warm-up steps, not instead of them."""
+    t_end = time.perf_counter() + SPINUP_MS * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(32):
+            fn()
+        ctx.sync()
+
+
 def time_launches(ctx, fn, steps, warmup):
     """-> (wall seconds for `steps` launches, HIP-event ms per launch)."""
+    spin_up(ctx, fn)
     for _ in range(warmup):
         fn()
     ctx.sync()
@@ -304,15 +322,19 @@ def bench_cnn(steps, warmup, with_cpu=True):
 
 
 def main():
+    global SPINUP_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--spinup-ms", type=float, default=SPINUP_MS,
+                    help="untimed launches of each measured kernel for this long before its warm-up steps (clock settling)")
     ap.add_argument("--no-extras", action="store_true", help="skip matvec and MLP measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain 256 MiB copy kernel (scale factor for rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
+    SPINUP_MS = max(0.0, args.spinup_ms)
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path shards over the dense-column axis "
                  "with no exchange: every GPU would take B/N of the batch against its own copy of the weights); run with --gpus 1")
@@ -347,7 +369,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "ellpack_matmul large FC: W 4096x4096 N(0,0.02) per-row top-10%% (r=410, nnz=%d), "
                                "X 4096x256 N(0,1), bias N(0,0.1), seed 45" % E.total_nnz,
-                   "m": E.m, "n": E.n, "r": E.r, "C": C, "sparsity": 0.9, "device": dev_name},
+                   "m": E.m, "n": E.n, "r": E.r, "C": C, "sparsity": 0.9, "device": dev_name,
+                   "spinup_ms": SPINUP_MS},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
                      "kernel": "ellpack_matmul_tiled_kernel", "kernel_us": round(ev_ms * 1e3, 2), "alg_bytes_per_launch": nbytes,
