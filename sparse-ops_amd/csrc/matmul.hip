@@ -195,6 +195,85 @@ void launch_act(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, c
 }
 
 // ---------------------------------------------------------------------------
+// Few rows (a classifier head): rows x column tiles give fewer waves than the chip
+// has CUs, so a wave's own gather latency is all there is to hide, and the bytes it
+// can keep in flight are bounded by its registers.  Here a workgroup of 16 waves
+// shares one (row, 64-column tile): the waves split the row's nonzeros among them
+// for the gathers (16 times the loads in flight), park the gathered X segments in
+// LDS in slot order, and the first wave then runs the multiply-adds over them in
+// slot order starting from the bias -- the same rounding sequence as the row kernel.
+// ---------------------------------------------------------------------------
+
+constexpr int kShareWaves = 16;
+constexpr int kSharePerWave = 32;                           // gathers per wave and chunk
+constexpr int kShareChunk = kShareWaves * kSharePerWave;    // slots per chunk: 128 KB of X segments
+constexpr size_t kShareLdsBytes = (size_t)kShareChunk * 64 * sizeof(float) + kShareChunk * sizeof(float);
+
+template <int ACT>
+__global__ __launch_bounds__(kShareWaves * 64)
+void ellpack_matmul_shared_gather_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
+                                         const uint32_t *__restrict__ nnz, uint32_t r,
+                                         const float *__restrict__ X, uint32_t C,
+                                         const float *__restrict__ bias, float *__restrict__ Y, uint32_t ntiles)
+{
+    extern __shared__ __attribute__((aligned(16))) float share_lds[];
+    float *xs = share_lds;                              // [kShareChunk][64]
+    float *ws = share_lds + (size_t)kShareChunk * 64;   // [kShareChunk]
+    const uint32_t tile = blockIdx.x % ntiles, row = blockIdx.x / ntiles;   // the grid is exactly m * ntiles
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t col = tile * 64u + lane;
+    const bool live = col < C;
+    const uint32_t cnt = nnz[row];
+    const float *__restrict__ wrow = Wd + (size_t)row * r;
+    const uint32_t *__restrict__ irow = idx + (size_t)row * r;
+    const float *__restrict__ xcol = X + (live ? col : 0u);
+    float acc = bias ? bias[row] : 0.0f;
+
+    for (uint32_t s0 = 0; s0 < cnt; s0 += kShareChunk) {
+        const uint32_t chunk = min((uint32_t)kShareChunk, cnt - s0);
+        const uint32_t w0 = wave * kSharePerWave;        // this wave gathers slots s0 + w0 .. + kSharePerWave
+        if (w0 < chunk) {
+            const uint32_t mine = min((uint32_t)kSharePerWave, chunk - w0);
+            float x[kSharePerWave];
+#pragma unroll
+            for (int u = 0; u < kSharePerWave; ++u) {    // slots past the wave's share re-read its last one
+                const uint32_t j = s0 + w0 + min((uint32_t)u, mine - 1u);
+                x[u] = xcol[(size_t)irow[j] * C];
+            }
+            if (lane < mine) ws[w0 + lane] = wrow[s0 + w0 + lane];
+#pragma unroll
+            for (int u = 0; u < kSharePerWave; ++u)
+                if ((uint32_t)u < mine) xs[(w0 + u) * 64u + lane] = x[u];
+        }
+        __syncthreads();
+        if (wave == 0) {
+            uint32_t s = 0;
+            for (; s + 8 <= chunk; s += 8) {
+                float w[8], x[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) { w[u] = ws[s + u]; x[u] = xs[(s + u) * 64u + lane]; }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) acc = __builtin_fmaf(w[u], x[u], acc);
+            }
+            for (; s < chunk; ++s) acc = __builtin_fmaf(ws[s], xs[s * 64u + lane], acc);
+        }
+        __syncthreads();                                  // the next chunk overwrites what wave 0 was reading
+    }
+    if (wave == 0 && live) Y[(size_t)row * C + col] = so_epilogue<ACT>(acc);
+}
+
+template <int ACT>
+so_status launch_shared_gather(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, const float *dBias, float *dY)
+{
+    SO_HIP(so_allow_big_lds(ctx, (const void *)ellpack_matmul_shared_gather_kernel<ACT>));
+    const uint32_t ntiles = so_ceil_div(C, 64u);
+    ellpack_matmul_shared_gather_kernel<ACT><<<E->m * ntiles, kShareWaves * 64, kShareLdsBytes, ctx->stream>>>(
+        E->d_Wd, E->d_idx, E->d_nnz, E->r, dX, C, dBias, dY, ntiles);
+    return SO_OK;
+}
+
+// ---------------------------------------------------------------------------
 // LDS-staged variant (SO_LAYOUT_TILED).
 //
 // The row kernel above moves every X operand through the vector L1, which
@@ -461,7 +540,23 @@ extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX
     // Few waves in total (at most one per SIMD even with one column per lane): the
     // launch is latency-bound, so spread it over as many waves as possible and give
     // each wave 2 x 32 gathers in flight.
-    if ((uint64_t)E->m * so_ceil_div(C, 64) <= 4ull * (uint64_t)ctx->compute_units && E->max_nnz >= 64)
+    const uint64_t row_tiles = (uint64_t)E->m * so_ceil_div(C, 64);
+    // At most one (row, tile) per CU and rows long enough to be worth sharing: 16 waves gather for each.
+    bool share = row_tiles <= (uint64_t)ctx->compute_units && E->max_nnz >= 128 && (size_t)ctx->max_lds_bytes >= kShareLdsBytes;
+    if (ctx->tune.matmul_share >= 0) share = share && ctx->tune.matmul_share == 1;
+    if (share) {
+        so_status st;
+        switch (act) {
+        case SO_ACT_RELU:    st = launch_shared_gather<SO_ACT_RELU>(ctx, E, dX, C, dBias, dY); break;
+        case SO_ACT_SIGMOID: st = launch_shared_gather<SO_ACT_SIGMOID>(ctx, E, dX, C, dBias, dY); break;
+        case SO_ACT_TANH:    st = launch_shared_gather<SO_ACT_TANH>(ctx, E, dX, C, dBias, dY); break;
+        default:             st = launch_shared_gather<SO_ACT_NONE>(ctx, E, dX, C, dBias, dY); break;
+        }
+        if (st != SO_OK) return st;
+        SO_LAUNCH_CHECK();
+        return SO_OK;
+    }
+    if (row_tiles <= 4ull * (uint64_t)ctx->compute_units && E->max_nnz >= 64)
         launch_act<1, 32>(ctx, E, dX, C, dBias, dY, act);
     else if (vec == 4) launch_act<4>(ctx, E, dX, C, dBias, dY, act);
     else if (vec == 2) launch_act<2>(ctx, E, dX, C, dBias, dY, act);

@@ -56,6 +56,7 @@ static void read_tuning(so_tuning &t)
     t = so_tuning();
     t.matmul_tiled = env_int("SPARSEOPS_MATMUL_TILED", -1);
     t.matmul_vec = env_int("SPARSEOPS_MATMUL_VEC", 0);
+    t.matmul_share = env_int("SPARSEOPS_MATMUL_SHARE", -1);
     const int lanes = env_int("SPARSEOPS_MATVEC_LANES", 0);
     t.matvec_lanes = (lanes == 8 || lanes == 16 || lanes == 32 || lanes == 64) ? lanes : 0;
     t.conv_window = env_int("SPARSEOPS_CONV_WINDOW", -1);

@@ -177,6 +177,37 @@ def test_matmul_lds_tiled_keeps_negative_zero(ctx, oracle):
         assert np.array_equal(Y, Yo) and np.array_equal(np.signbit(Y), np.signbit(Yo))
 
 
+@pytest.mark.parametrize("m,n,C,sp", [(1, 1000, 32, .1), (3, 5000, 100, .8), (10, 4096, 256, .9), (2, 3000, 64, 0.),
+                                      (7, 700, 132, .3), (4, 200, 64, .1), (5, 6000, 20, .5), (1, 130, 1, 0.),
+                                      (1, 513, 64, 0.), (2, 1025, 70, 0.)])
+@pytest.mark.parametrize("act", ["none", "relu", "tanh"])
+def test_matmul_few_rows_shared_gather(ctx, oracle, m, n, C, sp, act):
+    """At most one (row, 64-column tile) per CU and rows of 128 nonzeros or more: the 16 waves of a
+    workgroup gather one row's X segments into LDS and its first wave accumulates them in slot
+    order.  Rows longer than one 512-slot chunk, rows that end inside a wave's share, an empty
+    row, a partial column tile, an infinite X entry next to slots that must not be read."""
+    rng = np.random.default_rng(m * 131 + n + C)
+    W = sparse_matrix(rng, m, n, sp)
+    if m > 2:
+        W[1] = 0
+    X = rng.standard_normal((n, C)).astype(np.float32)
+    X[0, 0] = np.inf
+    b = rng.standard_normal(m).astype(np.float32)
+    E = datagen.encode_dense(W)
+    assert E.nnz.max() >= 128
+    results = []
+    for share in ("1", "0"):           # "0": the same launch on the row kernel
+        with ctx.tuning(SPARSEOPS_MATMUL_SHARE=share):
+            for bias in (b, None):
+                Y, Yo = _gpu_matmul(ctx, E, X, bias, act, hipabi.LAYOUT_ROW), oracle.matmul(as_oracle(E), X, bias, act)
+                if act == "tanh":
+                    assert rel_err(Y[np.isfinite(Yo)], Yo[np.isfinite(Yo)]) <= ACT_TOL
+                else:
+                    assert np.array_equal(Y, Yo, equal_nan=True)
+                results.append(Y)
+    assert np.array_equal(results[0], results[2], equal_nan=True) and np.array_equal(results[1], results[3], equal_nan=True)
+
+
 def test_matmul_degenerate_shapes(ctx, oracle):
     # zero-sized launches are early-outs, not HIP errors
     for (m, n, C) in [(0, 0, 0), (0, 5, 3), (5, 0, 3), (5, 4, 0)]:

@@ -76,13 +76,17 @@ def test_mlp_graph_and_eager_agree(backend, tmp_path):
           datagen.magnitude_prune(rng.standard_normal((20, 80)).astype(np.float32), .8)]
     path = ow.save(str(tmp_path / "m.onnx"), ow.mlp_model(Ws, ["Relu", "Tanh"], 32))
     X = rng.standard_normal((32, 60)).astype(np.float32)
-    Yg = backend.SparseOnnxModel(path).run(X)
-    os.environ["SPARSEOPS_NO_GRAPH"] = "1"
-    try:
-        Ye = backend.SparseOnnxModel(path).run(X)
-    finally:
-        del os.environ["SPARSEOPS_NO_GRAPH"]
-    assert np.array_equal(Yg, Ye)
+    Yd = backend.SparseOnnxModel(path).run(X)      # the library's own choice (short chain: no graph)
+    results = {}
+    for no_graph in ("0", "1"):                    # "0": always record a launch graph, "1": never
+        os.environ["SPARSEOPS_NO_GRAPH"] = no_graph
+        try:
+            model = backend.SparseOnnxModel(path)
+            results[no_graph] = [model.run(X) for _ in range(3)]      # replays too
+        finally:
+            del os.environ["SPARSEOPS_NO_GRAPH"]
+    for Y in results["0"] + results["1"]:
+        assert np.array_equal(Y, Yd)
 
 
 def test_mlp_config4(backend, oracle, tmp_path):
