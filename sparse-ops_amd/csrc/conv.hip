@@ -15,6 +15,7 @@
 // the CU's L1.  Accumulation is bias first, then one fused multiply-add per stored
 // nonzero in ascending slot order, as in the reference.
 #include "so_internal.h"
+#include "dpp_steps.h"
 
 #include <algorithm>
 #include <cstdlib>
@@ -255,10 +256,12 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
 // entries each), so a wave covers 64/LPP pixels; the 16 waves are PG pixel groups x CG channel
 // groups and a wave accumulates CPW output channels.  The batch tile is 16 (LPP = 4): measured
 // against 32 and 8 it was the fastest on every layer of the ResNet-18-shaped stack, because the
-// smaller window lets a chunk hold twice the channels (longer runs per channel, half the barriers).  Entries are wave-uniform: they arrive
-// through scalar loads, four at a time and one quad ahead, so the weight is a scalar operand
-// of the multiply-adds and the tap offset a scalar addend of the LDS address (handing them
-// round with v_readlane was measured at three plain VALU slots per value).  Per output the
+// smaller window lets a chunk hold twice the channels (longer runs per channel, half the barriers).  Entries are wave-uniform.  With
+// 8 channels per wave they arrive through scalar loads, four at a time and one quad ahead, so
+// the weight is a scalar operand of the multiply-adds and the tap offset a scalar addend of the
+// LDS address; with fewer channels per wave (fewer, longer runs and usually fewer waves to hide
+// a scalar load behind) they are held one per lane and handed round by DPP (dpp_steps.h), 16
+// entries per vector load, one group ahead.  Per output the
 // multiply-adds run in slot order (chunks ascend, slots ascend inside a chunk): same bits as
 // the kernel above.  Windows are double-buffered: chunk t+1 is fetched into registers while
 // chunk t is computed.
@@ -361,8 +364,23 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
     // stream ends with a padding quad, so the request after the last quad is harmless.
     const int4 *__restrict__ sp = stream + 2 * (size_t)gbase[gi];
     const uint32_t *__restrict__ qp = quads + (size_t)gi * a.nch * CPW;
-    int4 cur0 = sp[0], cur1 = sp[1];
-    sp += 2;
+    int4 cur0 = make_int4(0, 0, 0, 0), cur1 = cur0;
+    // LANE_ENT: the entries sit in lanes instead (lane l of every 16-lane row holds entry l of the
+    // next 16), fetched with vector loads one group ahead and broadcast by DPP: vector loads have
+    // their own counter, so waiting for LDS data never waits for entries, which is what bounds the
+    // scalar path when there are too few waves to hide the scalar loads' latency.  Measured on a
+    // ResNet-18-shaped stack: 5-11 % faster per layer with 1 or 2 channels per wave, equal with 4,
+    // 9 % slower with 8 (batch 32); 8-13 % faster over the whole stack at batches 1 to 16.
+    constexpr bool LANE_ENT = CPW < 8;
+    const int2 *__restrict__ ep = reinterpret_cast<const int2 *>(sp) + (lane & 15u);
+    int2 ecur = make_int2(0, 0);
+    if constexpr (LANE_ENT) {
+        ecur = ep[0];
+    } else {
+        cur0 = sp[0];
+        cur1 = sp[1];
+        sp += 2;
+    }
     __syncthreads();
 
     const char *lds_bytes = reinterpret_cast<const char *>(win_lds);
@@ -376,6 +394,16 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
         for (int c = 0; c < CPW; ++c) nq[c] = computes ? qp[t * CPW + c] : 0u;
 #pragma unroll
         for (int c = 0; c < CPW; ++c) {
+            if constexpr (LANE_ENT) {
+                for (uint32_t q = 0; q < nq[c]; q += 4u) {
+                    const uint32_t steps = 4u * min(4u, nq[c] - q);      // this group: 4, 8, 12 or 16 entries
+                    ep += steps;
+                    const int2 enxt = ep[0];                              // the stream ends with 16 padding entries
+                    so_dpp::tiled_chunk(lds_bytes + base, __int_as_float(ecur.x), (uint32_t)ecur.y << SHIFT, steps, acc[c]);
+                    ecur = enxt;
+                }
+                continue;
+            }
             for (uint32_t q = 0; q < nq[c]; ++q) {
                 const int4 nxt0 = sp[0], nxt1 = sp[1];
                 sp += 2;
@@ -637,7 +665,8 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     const float neg_zero = -0.0f;
     uint32_t pad_bits;
     std::memcpy(&pad_bits, &neg_zero, 4);
-    std::vector<int2> stream((size_t)(total_quads + 1) * 4, make_int2((int32_t)pad_bits, (int32_t)(cc * w.IH * w.IW)));
+    // four padding quads at the end: the kernels request entries one quad, or one group of 16, ahead
+    std::vector<int2> stream((size_t)(total_quads + 4) * 4, make_int2((int32_t)pad_bits, (int32_t)(cc * w.IH * w.IW)));
     {
         size_t pos = 0;                                            // entries written so far
         std::vector<uint32_t> next(E->m, 0);                       // next unread slot of every row
