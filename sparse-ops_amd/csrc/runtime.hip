@@ -325,7 +325,7 @@ static so_status build_tiled(so_ctx *ctx, so_ellpack *E, const float *Wd, const 
     std::stable_sort(order.begin(), order.end(), longer_first);
     for (uint32_t b0 = 0; b0 < m; b0 += 64)
         std::stable_sort(blockwise.begin() + b0, blockwise.begin() + std::min(m, b0 + 64), longer_first);
-    {
+    if ((uint64_t)m * T.ntiles <= (1ull << 28)) {                     // the comparison needs 2 bytes per (row, tile)
         std::vector<uint16_t> per_tile((size_t)m * T.ntiles, 0);      // a tile has at most 256 columns
         for (uint32_t i = 0; i < m; ++i)
             for (uint32_t k = 0; k < nnz[i]; ++k) ++per_tile[(size_t)i * T.ntiles + idx[(size_t)i * r + k] / KT];
