@@ -59,6 +59,7 @@ static void read_tuning(so_tuning &t)
     t.matmul_share = env_int("SPARSEOPS_MATMUL_SHARE", -1);
     const int lanes = env_int("SPARSEOPS_MATVEC_LANES", 0);
     t.matvec_lanes = (lanes == 8 || lanes == 16 || lanes == 32 || lanes == 64) ? lanes : 0;
+    t.conv_min_cg = env_int("SPARSEOPS_CONV_MIN_CG", 0);
     t.conv_window = env_int("SPARSEOPS_CONV_WINDOW", -1);
     t.conv_cpw = env_int("SPARSEOPS_CONV_CPW", 0);
     t.conv_tilepx = env_int("SPARSEOPS_CONV_TILEPX", 0);

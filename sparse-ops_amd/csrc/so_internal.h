@@ -15,6 +15,7 @@ struct so_tuning {
     int matmul_vec = 0;      // SPARSEOPS_MATMUL_VEC: 1 or 2 columns per lane at most
     int matmul_share = -1;   // SPARSEOPS_MATMUL_SHARE: 0 forbids the shared-gather kernel for few-row launches
     int matvec_lanes = 0;    // SPARSEOPS_MATVEC_LANES: 8, 16, 32 or 64 lanes per row
+    int conv_min_cg = 0;     // SPARSEOPS_CONV_MIN_CG: fewest channel groups per workgroup a small grid may shrink to (16: never shrink)
     int conv_window = -1;    // SPARSEOPS_CONV_WINDOW: 1 forces the LDS-windowed kernel, 0 forbids it
     int conv_cpw = 0;        // SPARSEOPS_CONV_CPW: most output channels per wave
     int conv_tilepx = 0;     // SPARSEOPS_CONV_TILEPX: most output pixels per tile
