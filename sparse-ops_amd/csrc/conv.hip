@@ -613,7 +613,12 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     // At most 32 output pixels per tile; 16 for small images (up to 16 x 16 output pixels), where the
     // smaller window lets a chunk hold more channels and the extra tiles give the chip more workgroups
     // (measured: 14 x 14 layer 79 -> 71 us, 7 x 7 layer 89 -> 81 us; 28 x 28 and 56 x 56 lose 8-25 %).
+    // Those sizes are for the batch tile of 16 (4 lanes per pixel).  A batch tile of 8 or 4 puts 2 or
+    // 4 times the pixels on a wave's 64 lanes and in the same LDS: the tile is then one wave of
+    // pixels, 32 or 64 (measured on the stack at batch 1: 0.478 -> 0.416 ms; at batch 8: 0.549 -> 0.523).
+    const uint32_t lpp_for_batch = window_lpp(batch) ? window_lpp(batch) : kWinLPP;
     uint32_t max_px = (uint64_t)g.H_out * g.W_out <= 256 ? 16u : 32u;
+    if (lpp_for_batch < kWinLPP) max_px = 64u / lpp_for_batch;
     if (ctx->tune.conv_tilepx > 0) max_px = (uint32_t)ctx->tune.conv_tilepx;
     for (uint32_t th = 1; th <= max_px && th <= g.H_out; ++th)
         for (uint32_t tw = 1; th * tw <= max_px && tw <= g.W_out; ++tw) {
@@ -636,7 +641,7 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     // Both depend on the batch tile (16, 8 or 4 entries): a smaller tile lets a chunk hold more
     // channels, i.e. fewer chunks, fewer barriers and longer runs -- what small batches, whose
     // launches are bound by latency, need.  A layout sized for a batch tile also serves smaller ones.
-    w.lpp = window_lpp(batch) ? window_lpp(batch) : kWinLPP;
+    w.lpp = lpp_for_batch;
     const uint64_t px_bytes = w.lpp * 16, lds_budget = (uint64_t)ctx->max_lds_bytes;
     uint32_t cc = g.Cin;
     while (cc > 0 && ((cc < g.Cin ? 2ull : 1ull) * (cc + 1) * w.IH * w.IW * px_bytes > lds_budget ||

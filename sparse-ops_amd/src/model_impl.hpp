@@ -57,8 +57,8 @@ struct SparseOnnxModel::Impl {
     int input_slot = -1, output_slot = -1;
     std::size_t in_features = 0, out_features = 0;
     uint32_t batch = 0;            // samples per call, as the caller sees it
-    uint32_t pbatch = 0;           // samples per row of every arena tensor: batch rounded up to a multiple of four when
-                                   // the model has convolutions (their LDS-windowed kernel works on batch tiles of 4+)
+    uint32_t pbatch = 0;           // samples per row of every arena tensor: batch rounded up to 4, 8 or a multiple of 16
+                                   // when the model has convolutions (their LDS-windowed kernel works on such batch tiles)
     bool has_conv = false;
 
     sparseops::DeviceBuffer bias_pool;   // all biases, contiguous

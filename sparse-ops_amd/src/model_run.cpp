@@ -21,10 +21,13 @@ void SparseOnnxModel::resize_buffers(uint32_t batch)
     if (M.graph) { so_graph_free(ctx, M.graph); M.graph = nullptr; }
     M.has_conv = false;
     for (const LayerPlan &L : M.layers) M.has_conv |= L.conv != nullptr;
-    // A batch that is not a multiple of four would push every convolution onto the slower
-    // gather kernel: carry it in rows of the next multiple of four instead (the extra columns are
-    // zeros on input and are never copied out; batch entries do not interact).
-    const uint32_t pbatch = (M.has_conv && batch % 4 != 0) ? (batch + 3u) / 4u * 4u : batch;
+    // The convolutions work on batch tiles of 16, 8 or 4 entries, and the larger the tile the less a
+    // batch entry costs: a batch is carried in rows of 4 (up to 4 entries), 8 (up to 8) or the next
+    // multiple of 16 (the extra columns are zeros on input and are never copied out; batch entries
+    // do not interact).  Measured on a ResNet-18-shaped stack: 12 entries as 12 0.86 ms, as 16
+    // 0.76 ms; 24 as 24 1.31 ms, as 32 1.24 ms.
+    uint32_t pbatch = batch;
+    if (M.has_conv) pbatch = batch <= 4 ? 4u : batch <= 8 ? 8u : (batch + 15u) / 16u * 16u;
     // Slot offsets for this batch, 256-byte aligned.
     std::size_t total = 0;
     std::size_t widest = std::max(M.in_features, M.out_features);

@@ -153,7 +153,7 @@ def oracle_cnn(oracle, t, X):
     return oracle.matmul(oracle.encode(t["Wf"]), g1, t["bf"], "relu").T
 
 
-@pytest.mark.parametrize("B", [4, 32])
+@pytest.mark.parametrize("B", [1, 4, 7, 9, 12, 20, 32])      # carried in rows of 4, 4, 8, 16, 16, 32, 32 entries
 def test_cnn(backend, oracle, tmp_path, B):
     rng = np.random.default_rng(8 + B)
     payload, t = cnn_model(rng, B)
