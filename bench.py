@@ -442,7 +442,7 @@ def main():
         log("sparse MLP ...")
         extras["mlp"] = bench_mlp(k, args.warmup, with_cpu=not args.no_cpu)
         log("sparse CNN ...")
-        extras["cnn"] = bench_cnn(max(5, args.steps // 20), 2, with_cpu=not args.no_cpu)
+        extras["cnn"] = bench_cnn(max(10, args.steps // 10), 5, with_cpu=not args.no_cpu)
         result["extras"] = extras
     ctx.close()
     print(json.dumps(result), flush=True)
