@@ -209,15 +209,15 @@ so_status so_act(so_ctx *ctx, int act, const float *dX, size_t len, float *dY);
 so_status so_transpose(so_ctx *ctx, const float *dSrc, uint32_t rows, uint32_t cols, float *dDst);
 /* Copy a [rows x cols] matrix between buffers whose rows start src_stride / dst_stride floats
  * apart; with zero_fill the rest of every destination row (cols .. dst_stride) is set to zero.
- * No counterpart in the reference: the model runtime uses it to carry a batch that is not a
- * multiple of four inside buffers that are (what the convolution kernels' batch tiles need). */
+ * No counterpart in the reference: the model runtime uses it to carry a batch inside buffers whose
+ * rows hold 4, 8 or a multiple of 16 entries (what the convolution kernels' batch tiles need). */
 so_status so_copy_rows(so_ctx *ctx, const float *dSrc, size_t src_stride, uint32_t rows, uint32_t cols,
                        float *dDst, size_t dst_stride, int zero_fill);
 
 /* ---- launch graphs -------------------------------------------------------
  * Record every launch made on the context between begin and end into one
  * hipGraph, then replay it with a single submission (SparseOnnxModel::run uses
- * this for the layer chain, src/model_run.cpp:28-127).  No allocation, copy to
+ * this for layer chains of eight layers or more, src/model_run.cpp:28-127).  No allocation, copy to
  * or from the host, or timer call may happen while recording. */
 typedef struct so_graph so_graph;
 so_status so_graph_begin(so_ctx *ctx);
