@@ -148,6 +148,50 @@ def test_conv_plan_tune_changes_layout_not_results(ctx, oracle):
     dE.free()
 
 
+@pytest.mark.parametrize("Cin,Cout,H,Wi,s", [(128, 96, 7, 7, 1), (64, 80, 14, 14, 1), (40, 48, 28, 28, 1), (48, 64, 15, 13, 2)])
+@pytest.mark.parametrize("B", [4, 8, 16])
+def test_conv_plan_tuned_for_small_batches(ctx, oracle, Cin, Cout, H, Wi, s, B):
+    """A plan tuned for a batch tile of 4 or 8 takes pixel tiles of a whole wave (64 or 32 pixels)
+    and, on small images, fewer computing waves per workgroup; entries are held in lanes.  Deep
+    layers on small images, several channel chunks, an empty and a dense output channel."""
+    from oracle import conv_geom as ocg
+    rng = np.random.default_rng(Cin + Cout * 7 + H * 31 + B)
+    Wc = sparse_matrix(rng, Cout, Cin * 9, .8)
+    Wc[5] = 0
+    Wc[Cout - 1] = rng.standard_normal(Cin * 9)
+    E = datagen.encode_dense(Wc)
+    g, og = hipabi.conv_geom(Cin, Cout, 3, 3, H, Wi, (s, s), (1, 1)), ocg(Cin, Cout, 3, 3, H, Wi, (s, s), (1, 1))
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+    plan = ctx.conv_plan(dE, g)
+    ctx.conv_plan_tune(plan, B)
+    win = ctx.conv_plan_window(plan)
+    assert win is not None
+    X = rng.standard_normal((Cin, H, Wi, B)).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    R = rng.standard_normal((Cout, g.H_out, g.W_out, B)).astype(np.float32)
+    Yo = oracle.conv2d_pf(as_oracle(E), og, X, B, b, "none")
+    with ctx.tuning(SPARSEOPS_CONV_WINDOW="1"):
+        assert np.array_equal(_conv_keep_plan(ctx, plan, g, X, B, b, "none"), Yo)
+        assert np.array_equal(_conv_keep_plan(ctx, plan, g, X, B, None, "relu"), oracle.conv2d_pf(as_oracle(E), og, X, B, None, "relu"))
+        assert np.array_equal(_conv_keep_plan(ctx, plan, g, X, B, b, "relu", R), oracle.act(oracle.add(Yo, R), "relu"))
+        with ctx.tuning(SPARSEOPS_CONV_MIN_CG="16"):          # the same launch without shrinking the channel groups
+            assert np.array_equal(_conv_keep_plan(ctx, plan, g, X, B, b, "none"), Yo)
+    ctx.conv_plan_free(plan)
+    dE.free()
+
+
+def _conv_keep_plan(ctx, plan, g, X, B, bias, act, residual=None):
+    dX, dY = ctx.array(X), ctx.empty((g.Cout, g.H_out, g.W_out, B))
+    dB = ctx.array(bias) if bias is not None else None
+    dR = ctx.array(residual) if residual is not None else None
+    ctx.conv2d(plan, dX, B, dB, dY, act, residual=dR)
+    Y = dY.download()
+    for a in (dX, dY, dB, dR):
+        if a is not None:
+            a.free()
+    return Y
+
+
 def test_conv_reference_vectors(ctx, golden):
     for i, c in enumerate(golden["conv_cases"]):
         Cin, Cout, H, Wi, B = (int(v) for v in c[:5])
