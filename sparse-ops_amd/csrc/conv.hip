@@ -278,7 +278,15 @@ struct WinArgs {
     uint32_t win_f4;    // float4 elements of one chunk's window
     uint32_t buf_f4;    // window plus the zero plane: stride between the two buffers
     uint32_t nbuf;      // 2: double-buffered windows; 1: a single chunk, nothing to overlap
+    uint32_t sth, stw;  // window pixels between neighbouring output pixels
+    uint32_t sbh, sbw;  // input pixels between neighbouring window pixels
 };
+
+// Along an axis on which the kernel has a single tap, a strided convolution reads only every
+// stride-th input pixel: the window then holds just those (one window pixel per output pixel)
+// instead of all the pixels in between.
+inline uint32_t window_step(uint32_t k, uint32_t stride) { return k == 1 ? 1u : stride; }
+inline uint32_t window_subsample(uint32_t k, uint32_t stride) { return k == 1 ? stride : 1u; }
 
 template <int CPW, int LPP, int ACT>
 __global__ __launch_bounds__(kWinThreads)
@@ -305,7 +313,7 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
     const uint32_t pc = pvalid ? pl : 0u;
     const uint32_t ty = pc / a.TW, tx = pc % a.TW;
     const bool live = computes && pvalid && th0 + ty < g.H_out && tw0 + tx < g.W_out;
-    const uint32_t lanebase = ((ty * g.stride_h * a.IW + tx * g.stride_w) << SHIFT) + b4 * 16u;   // bytes
+    const uint32_t lanebase = ((ty * a.sth * a.IW + tx * a.stw) << SHIFT) + b4 * 16u;   // bytes
     const uint32_t buf_bytes = a.buf_f4 * 16u;
 
     // window elements this thread copies: element e = tid + k*1024 is float4 (cl, ih, iw, b4)
@@ -319,8 +327,8 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
         if (e < a.win_f4) {
             const uint32_t eb = e % LPP, px = e / LPP;
             const uint32_t iw = px % a.IW, rest = px / a.IW, ih = rest % a.IH, cl = rest / a.IH;
-            const int32_t gh = (int32_t)(th0 * g.stride_h + ih) - (int32_t)g.pad_h;
-            const int32_t gw = (int32_t)(tw0 * g.stride_w + iw) - (int32_t)g.pad_w;
+            const int32_t gh = (int32_t)(th0 * g.stride_h + ih * a.sbh) - (int32_t)g.pad_h;
+            const int32_t gw = (int32_t)(tw0 * g.stride_w + iw * a.sbw) - (int32_t)g.pad_w;
             gcl[k] = cl;
             if ((uint32_t)gh < g.H_in && (uint32_t)gw < g.W_in)
                 goff[k] = (int32_t)(((cl * g.H_in + (uint32_t)gh) * g.W_in + (uint32_t)gw) * B + bz + eb * 4u);
@@ -530,6 +538,8 @@ so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, 
     a.win_f4 = w.cc * w.IH * w.IW * LPP;
     a.buf_f4 = (w.cc + 1) * w.IH * w.IW * LPP;
     a.nbuf = w.nch > 1 ? 2u : 1u;
+    a.sth = window_step(plan->g.kH, plan->g.stride_h); a.stw = window_step(plan->g.kW, plan->g.stride_w);
+    a.sbh = window_subsample(plan->g.kH, plan->g.stride_h); a.sbw = window_subsample(plan->g.kW, plan->g.stride_w);
     const size_t lds = (size_t)a.nbuf * a.buf_f4 * 16;
     // a layout whose chunks were sized for a smaller batch tile than this batch's does not fit
     if (LPP > w.lpp && (lds > (size_t)ctx->max_lds_bytes || a.win_f4 > (uint32_t)kWinMaxPerThread * kWinThreads)) return SO_OK;
@@ -623,8 +633,8 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     for (uint32_t th = 1; th <= max_px && th <= g.H_out; ++th)
         for (uint32_t tw = 1; th * tw <= max_px && tw <= g.W_out; ++tw) {
             const uint64_t tiles = (uint64_t)so_ceil_div(g.H_out, th) * so_ceil_div(g.W_out, tw);
-            const uint64_t win = (uint64_t)((th - 1) * g.stride_h + (g.kH - 1) * g.dil_h + 1) *
-                                 ((tw - 1) * g.stride_w + (g.kW - 1) * g.dil_w + 1);
+            const uint64_t win = (uint64_t)((th - 1) * window_step(g.kH, g.stride_h) + (g.kH - 1) * g.dil_h + 1) *
+                                 ((tw - 1) * window_step(g.kW, g.stride_w) + (g.kW - 1) * g.dil_w + 1);
             if (tiles < best_tiles || (tiles == best_tiles && win < best_win)) {
                 best_tiles = tiles; best_win = win; bestTH = th; bestTW = tw;
             }
@@ -632,8 +642,8 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     if (bestTH == 0) return SO_OK;
     so_conv_window w;
     w.TH = bestTH; w.TW = bestTW;
-    w.IH = (w.TH - 1) * g.stride_h + (g.kH - 1) * g.dil_h + 1;
-    w.IW = (w.TW - 1) * g.stride_w + (g.kW - 1) * g.dil_w + 1;
+    w.IH = (w.TH - 1) * window_step(g.kH, g.stride_h) + (g.kH - 1) * g.dil_h + 1;
+    w.IW = (w.TW - 1) * window_step(g.kW, g.stride_w) + (g.kW - 1) * g.dil_w + 1;
     w.tiles_y = so_ceil_div(g.H_out, w.TH);
     w.tiles_x = so_ceil_div(g.W_out, w.TW);
     if ((uint64_t)w.IH * w.IW > 4096) return SO_OK;

@@ -77,6 +77,10 @@ WINDOW_CASES = [
     (9, 21, 13, 11, 24, (3, 3), (2, 2), (1, 1), (1, 1), .5),      # batch 24 = 3 tiles of 8
     (16, 24, 30, 30, 4, (3, 3), (1, 1), (1, 1), (1, 1), .6),      # batch tile 4 (half the lanes of a wave idle)
     (3, 64, 32, 32, 12, (7, 7), (2, 2), (3, 3), (1, 1), .7),      # batch 12 = 3 tiles of 4
+    (64, 48, 28, 28, 32, (1, 1), (2, 2), (0, 0), (1, 1), .5),     # 1x1 stride 2 (a ResNet projection): the window holds every second pixel only
+    (32, 40, 15, 13, 8, (1, 1), (2, 3), (0, 0), (1, 1), .3),      # 1x1, strides 2 and 3, ragged tiles
+    (16, 24, 20, 20, 16, (1, 3), (2, 2), (0, 1), (1, 1), .5),     # one tap along h only: subsampled rows, full columns
+    (16, 24, 21, 20, 4, (3, 1), (2, 2), (1, 0), (1, 1), .5),      # and the other way round, batch tile 4
 ]
 
 
