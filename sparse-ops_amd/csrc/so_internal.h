@@ -53,6 +53,7 @@ struct so_tile_entry { float w; uint32_t off; };
 struct so_tile_info { uint32_t chunk0; uint32_t steps; };   // steps is a multiple of 4
 struct so_tiled {
     static constexpr uint32_t kTileRows = 256;   // X rows per LDS tile
+    static constexpr uint32_t kWavesPerGroup = 16;   // quads (waves) per workgroup of the kernel
     static constexpr uint32_t kSlabCols = 64;    // dense columns per workgroup
     static constexpr uint32_t kTileBytes = kTileRows * kSlabCols * 4;
     static constexpr uint32_t kZeroRowOff = 2 * kTileBytes;      // after the two tile buffers
@@ -84,6 +85,10 @@ struct so_graph {
 };
 
 void so_set_error(const char *fmt, ...);
+
+// csrc/matmul_tiled.hip: launches the LDS-staged kernel on E's TILED copy (the caller has checked that it applies).
+so_status so_matmul_tiled_launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
+                                 const float *dBias, float *dY, int act);
 
 // Kernels that ask for more than 48 KB of dynamic LDS must be told so once per device: this does
 // it the first time `kernel` is seen on the context's device (hipSuccess when already done).
