@@ -119,7 +119,13 @@ so_status so_timer_end(so_ctx *ctx, float *ms);
  * Wd[m*r], idx[m*r], nnz[m]).  Validates nnz[i] <= r and idx < n for every stored
  * slot (the reference validates only in a benchmark,
  * benchmark-mkl/matvec/bench_matvec.cpp:83-98) and fails with SO_ERR_BOUNDS.
- * `layouts` is a mask of SO_LAYOUT_*; ROW is always kept.  m, n or r may be 0. */
+ * `layouts` is a mask of SO_LAYOUT_*; ROW is always kept.  m, n or r may be 0.
+ * Column order inside a row: the encoder stores a row's columns strictly ascending
+ * (src/ellpack_encoder.cpp:28-41) and the TILED layout and the convolution's LDS-windowed layout
+ * rely on it.  Rows in any other order (or with a repeated column) are accepted, as the
+ * reference's kernels accept them: TILED is then not built (so_ellpack_dims reports the layouts
+ * kept), convolution plans on the handle use the gather kernel, and every kernel multiplies in
+ * slot order.  so_ellpack_decode needs distinct columns per row. */
 so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint32_t *idx,
                             const uint32_t *nnz, uint32_t m, uint32_t n, uint32_t r,
                             int layouts, so_ellpack **out);

@@ -45,6 +45,7 @@ struct so_conv_window {
 
 struct so_conv_plan {
     uint32_t tuned_batch = 32;   // batch the windowed layout was sized for
+    uint32_t tried_lpp = 0;      // lanes per pixel of the last attempt to build the windowed layout
     so_conv_geom g;
     const so_ellpack *E = nullptr;
     int2 *d_taps = nullptr;  // per slot: x = (cin*H + dh)*W + dw (elements of B floats), y = dh<<16 | (dw & 0xffff)
@@ -616,7 +617,9 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     const so_conv_geom &g = plan->g;
     const so_ellpack *E = plan->E;
     const uint32_t kHW = g.kH * g.kW;
+    plan->tried_lpp = window_lpp(batch) ? window_lpp(batch) : kWinLPP;
     if (kHW == 0 || E->r == 0 || E->total_nnz == 0) return SO_OK;
+    if (!E->ascending) return SO_OK;     // a chunk of input channels must be a slot range of every row
     // Tile: fewest tiles, then smallest window.
     uint32_t bestTH = 0, bestTW = 0;
     uint64_t best_tiles = ~0ull, best_win = ~0ull;
@@ -820,15 +823,20 @@ extern "C" so_status so_conv_plan_tune(so_ctx *ctx, so_conv_plan *plan, uint32_t
     SO_REQUIRE(ctx && plan, "so_conv_plan_tune: null argument");
     // The layout depends on the batch only through the number of batch tiles.
     const uint32_t batch = std::max(4u, B / 4u * 4u);
-    if (batch == plan->tuned_batch || plan->win.cc == 0) return SO_OK;
+    if (batch == plan->tuned_batch) return SO_OK;
     const so_ellpack *E = plan->E;
-    // Rebuild only if the batch changes the batch tile the chunks are sized for or the choice of
-    // channels per wave.
-    const double run = (double)E->total_nnz / (double)plan->g.Cout / plan->win.nch;
     const uint32_t lpp = window_lpp(batch) ? window_lpp(batch) : kWinLPP;
-    if (lpp == plan->win.lpp && choose_cpw(ctx, plan->win, plan->g.Cout, run, batch) == plan->win.cpw) {
-        plan->tuned_batch = batch;
-        return SO_OK;
+    // Rebuild only if the batch changes the batch tile the chunks are sized for or the choice of
+    // channels per wave.  A plan without the layout (the geometry did not suit the batch tile tried
+    // last) is tried again when the batch tile changes: a smaller tile holds more channels per chunk.
+    if (plan->win.cc == 0) {
+        if (lpp == plan->tried_lpp) { plan->tuned_batch = batch; return SO_OK; }
+    } else {
+        const double run = (double)E->total_nnz / (double)plan->g.Cout / plan->win.nch;
+        if (lpp == plan->win.lpp && choose_cpw(ctx, plan->win, plan->g.Cout, run, batch) == plan->win.cpw) {
+            plan->tuned_batch = batch;
+            return SO_OK;
+        }
     }
     const size_t slots = (size_t)E->m * E->r;
     std::vector<uint32_t> idx(slots), nnz(E->m);

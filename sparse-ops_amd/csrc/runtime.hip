@@ -411,8 +411,13 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
 
     // Validate on the host before anything reaches a kernel: every stored slot must
     // name a column inside X, every count must fit the row.
+    // The encoder stores a row's columns in strictly ascending order and the K-tiled matmul layout
+    // and the convolution's windowed layout walk a row on that assumption; a matrix filled in by
+    // hand in any other order (the reference's kernels take slots in whatever order they come) is
+    // served by the kernels that do the same, and the ordered layouts are not built for it.
     uint64_t total = 0;
     uint32_t max_nnz = 0;
+    bool ascending = true;
     for (uint32_t i = 0; i < m; ++i) {
         const uint32_t c = nnz[i];
         if (c > r) {
@@ -420,11 +425,13 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
             return SO_ERR_BOUNDS;
         }
         const uint32_t *row = idx + (size_t)i * r;
-        for (uint32_t k = 0; k < c; ++k)
+        for (uint32_t k = 0; k < c; ++k) {
             if (row[k] >= n) {
                 so_set_error("so_ellpack_upload: idx[%u,%u] = %u is not below n = %u", i, k, row[k], n);
                 return SO_ERR_BOUNDS;
             }
+            if (k > 0 && row[k] <= row[k - 1]) ascending = false;
+        }
         total += c;
         max_nnz = std::max(max_nnz, c);
     }
@@ -434,6 +441,8 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
     E->m = m; E->n = n; E->r = r;
     E->total_nnz = total;
     E->max_nnz = max_nnz;
+    E->ascending = ascending;
+    if (!ascending) layouts &= ~SO_LAYOUT_TILED;
     E->layouts = layouts | SO_LAYOUT_ROW;
 
     so_status s = upload_array(ctx, Wd, slots, &E->d_Wd);

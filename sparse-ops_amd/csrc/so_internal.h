@@ -69,6 +69,7 @@ struct so_ellpack {
     uint32_t m = 0, n = 0, r = 0;
     uint64_t total_nnz = 0;
     uint32_t max_nnz = 0;
+    bool ascending = true;       // every row's stored columns are strictly ascending (what the encoder produces)
     int layouts = 0;
     float *d_Wd = nullptr;       // [m*r] row-major
     uint32_t *d_idx = nullptr;   // [m*r]

@@ -8,7 +8,10 @@
 // code touching it still works, and never read by this library.
 //
 // Addition: `device`, the matrix's copy in GPU memory.  ellpack_matmul / ellpack_matvec create it
-// on first use; copies of the struct made afterwards share it.
+// on first use from the members as they are at that moment; copies of the struct made afterwards
+// share it.  The copy is not compared with the host arrays again: after writing to Wd, idx, nnz
+// (or m, n, r) of an Ellpack that has already been used, call invalidate_device(), and the next
+// kernel call uploads the members afresh.
 #pragma once
 
 #include <cstddef>
@@ -37,6 +40,8 @@ struct Ellpack {
     }
 
     std::size_t slots() const { return slot_count(m, r); }
+    /// Forget the GPU copy (this struct's reference to it): the next kernel call uploads again.
+    void invalidate_device() const { device.reset(); }
 
   private:
     static std::size_t slot_count(uint32_t rows, uint32_t per_row) { return std::size_t(rows) * per_row; }

@@ -24,7 +24,7 @@ def _product_step(E, bias):
 
 _ELEMENTWISE = {
     "Relu": lambda v: np.maximum(v, 0),
-    "Sigmoid": lambda v: (1 / (1 + np.exp(-v))).astype(np.float32),
+    "Sigmoid": lambda v: 1 / (1 + np.exp(-v)),
     "Tanh": np.tanh,
 }
 
@@ -34,17 +34,17 @@ class OnnxSparseModel:
         with open(onnx_path, "rb") as f:
             graph = onnx_wire.read_model(f.read())
         self._initializers = {name: arr.astype(np.float32) for name, arr in graph["initializers"].items()}
-        self.layers = []      # (name, Ellpack or None, bias or None), one per node: the reference's plan, for inspection
+        self.layers = []      # (op, Ellpack or None, bias or None, attrs), one per node: the reference's plan, same arity
         self._steps = []      # what run() calls, in order
         for node in graph["nodes"]:
             kind, operands = node["op_type"], node["input"]
             if kind in ("Gemm", "MatMul"):
                 E = encode(self._initializers[operands[1]])
                 bias = self._initializers[operands[2]] if kind == "Gemm" and len(operands) > 2 else None
-                self.layers.append(("matmul", E, bias))
+                self.layers.append(("matmul", E, bias, {}))
                 self._steps.append(_product_step(E, bias))
             elif kind in _ELEMENTWISE:
-                self.layers.append((kind.lower(), None, None))
+                self.layers.append((kind.lower(), None, None, {}))
                 self._steps.append(_ELEMENTWISE[kind])
             else:
                 raise NotImplementedError("Unsupported op %s" % kind)

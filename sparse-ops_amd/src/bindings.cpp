@@ -196,6 +196,15 @@ PYBIND11_MODULE(sparseops_backend, mod)
             }
             return py::array(Y);
         }, "Run inference on a (B, ...) input; returns the (B, ...) output")
+        .def("run_device", [](const SparseOnnxModel &model, std::uintptr_t d_input, uint32_t B, std::uintptr_t d_output) {
+            // Device pointers as integers (e.g. the .ptr of a ctypes-side allocation on the same
+            // device): [input_features x B] in, [output_features x B] out, both in HBM.  Waits for the
+            // chain, so the caller may read d_output from any stream afterwards.
+            py::gil_scoped_release nogil;
+            model.run_device(reinterpret_cast<const float *>(d_input), B, reinterpret_cast<float *>(d_output));
+            sparseops::check(so_sync(sparseops::context()), "so_sync");
+        }, py::arg("d_input"), py::arg("B"), py::arg("d_output"),
+           "Run the layer chain on device buffers ([features x B] row-major); no host copies")
         .def("resize_buffers", &SparseOnnxModel::resize_buffers, py::arg("batch"),
              "Pre-size every activation buffer for `batch` samples (run() then allocates nothing)")
         .def("output_shape", &SparseOnnxModel::output_shape)

@@ -70,7 +70,7 @@ struct SparseOnnxModel::Impl {
 
     ~Impl();
     float *slot_ptr(int s) const { return arena.f32() + slots[s].offset; }
-    void enqueue_layers(const float *in, float *out) const;  // in/out override the arena slots when non-null
+    void enqueue_layers() const;                             // one launch per layer, arena slot to arena slot
     void launch_chain() const;                               // graph replay or eager
     bool padded() const { return pbatch != batch; }
     void rows_in(const float *d_rows) const;                 // [in_features x batch] -> the input slot (rows padded with zeros)

@@ -46,7 +46,7 @@ void SparseOnnxModel::resize_buffers(uint32_t batch)
     if (M.use_graph && !M.layers.empty()) {
         check(so_graph_begin(ctx), "so_graph_begin");
         try {
-            M.enqueue_layers(nullptr, nullptr);
+            M.enqueue_layers();
         } catch (...) {
             so_graph *g = nullptr;
             so_graph_end(ctx, &g);
@@ -57,12 +57,15 @@ void SparseOnnxModel::resize_buffers(uint32_t batch)
     }
 }
 
-void SparseOnnxModel::Impl::enqueue_layers(const float *in, float *out) const
+void SparseOnnxModel::Impl::enqueue_layers() const
 {
     so_ctx *ctx = context();
     const uint32_t B = pbatch;
-    auto src = [&](int s) -> const float * { return (in && s == input_slot) ? in : slot_ptr(s); };
-    auto dst = [&](int s) -> float * { return (out && s == output_slot) ? out : slot_ptr(s); };
+    // Every layer reads and writes arena slots.  A slot id is shared by all tensors whose lifetimes
+    // do not overlap, so it identifies neither the graph input nor the graph output: callers' buffers
+    // are copied into the input slot before the chain and out of the output slot after it.
+    auto src = [&](int s) -> const float * { return slot_ptr(s); };
+    auto dst = [&](int s) -> float * { return slot_ptr(s); };
     for (const LayerPlan &L : layers) {
         const float *bias = L.has_bias ? bias_pool.f32() + L.bias_offset : nullptr;
         switch (L.op) {
@@ -94,7 +97,7 @@ void SparseOnnxModel::Impl::enqueue_layers(const float *in, float *out) const
 void SparseOnnxModel::Impl::launch_chain() const
 {
     if (graph) check(so_graph_launch(context(), graph), "so_graph_launch");
-    else enqueue_layers(nullptr, nullptr);
+    else enqueue_layers();
 }
 
 void SparseOnnxModel::Impl::rows_in(const float *d_rows) const
@@ -163,7 +166,10 @@ void SparseOnnxModel::run_device(const float *dInput, uint32_t B, float *dOutput
         M.rows_out(dOutput);
         return;
     }
-    M.enqueue_layers(dInput, dOutput);
+    so_ctx *ctx = context();
+    check(so_d2d(ctx, M.slot_ptr(M.input_slot), dInput, M.in_features * B * sizeof(float)), "so_d2d(input)");
+    M.launch_chain();
+    check(so_d2d(ctx, dOutput, M.slot_ptr(M.output_slot), M.out_features * B * sizeof(float)), "so_d2d(output)");
 }
 
 double SparseOnnxModel::time_device(int steps, int warmup) const

@@ -310,3 +310,33 @@ def test_launch_graph_replays(ctx, oracle):
         Yo = oracle.matmul(as_oracle(E2), oracle.matmul(as_oracle(E1), X, None, "relu"), None)
         assert np.array_equal(Y, Yo), it
     ctx.graph_free(g)
+
+
+def test_conv_rows_not_in_ascending_column_order(ctx, oracle):
+    """The windowed layout takes a chunk of input channels to be a slot range of every row; for weights
+    whose slots are in another order the plan carries no such layout, and the gather kernel computes the
+    convolution in slot order: bit-identical to the oracle on the shuffled arrays."""
+    from oracle import conv_geom as ocg
+    rng = np.random.default_rng(78)
+    Cin, Cout, H, Wi, B = 16, 24, 12, 12, 16
+    E = datagen.encode_dense(sparse_matrix(rng, Cout, Cin * 9, .6))
+    Wd, idx = E.Wd.copy(), E.idx.copy()
+    for i in range(E.m):
+        p = rng.permutation(int(E.nnz[i]))
+        Wd[i, :len(p)], idx[i, :len(p)] = E.Wd[i, p], E.idx[i, p]
+    Es = datagen.EllpackHost(E.m, E.n, E.r, Wd, idx, E.nnz)
+    g, og = hipabi.conv_geom(Cin, Cout, 3, 3, H, Wi, (1, 1), (1, 1)), ocg(Cin, Cout, 3, 3, H, Wi, (1, 1), (1, 1))
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+    plan = ctx.conv_plan(dE, g)
+    assert ctx.conv_plan_window(plan) is not None          # the sorted matrix gets the windowed layout
+    ctx.conv_plan_free(plan)
+    dE.free()
+    dE = ctx.upload_ellpack(Es.Wd, Es.idx, Es.nnz, Es.m, Es.n, Es.r)
+    plan = ctx.conv_plan(dE, g)
+    assert ctx.conv_plan_window(plan) is None
+    ctx.conv_plan_tune(plan, 8)
+    assert ctx.conv_plan_window(plan) is None
+    X = rng.standard_normal((Cin, H, Wi, B)).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    Y = _gpu_conv(ctx, dE, plan, g, X, B, b, "relu")
+    assert np.array_equal(Y, oracle.conv2d_pf(as_oracle(Es), og, X, B, b, "relu"))

@@ -347,3 +347,33 @@ def test_device_encoder_degenerate(ctx):
     assert dE.r == 0 and np.array_equal(dE.decode(), np.zeros((6, 70), np.float32))
     dZ.free()
     dE.free()
+
+
+def _shuffle_slots(E, rng):
+    """The same matrix with every row's stored slots in a random order (as a caller filling the
+    struct by hand might leave them); the reference's kernels take slots in whatever order they come."""
+    Wd, idx = E.Wd.copy(), E.idx.copy()
+    for i in range(E.m):
+        p = rng.permutation(int(E.nnz[i]))
+        Wd[i, :len(p)], idx[i, :len(p)] = E.Wd[i, p], E.idx[i, p]
+    return datagen.EllpackHost(E.m, E.n, E.r, Wd, idx, E.nnz)
+
+
+def test_matmul_rows_not_in_ascending_column_order(ctx, oracle):
+    """The K-tiled layout walks a row's columns in ascending order; for a matrix whose slots are in
+    another order it is not built (the handle reports ROW only) and so_matmul still multiplies in
+    slot order, like the reference: bit-identical to the oracle on the shuffled arrays."""
+    rng = np.random.default_rng(77)
+    E = _shuffle_slots(datagen.encode_dense(sparse_matrix(rng, 200, 700, .8)), rng)
+    X = rng.standard_normal((700, 64)).astype(np.float32)
+    b = rng.standard_normal(200).astype(np.float32)
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, TILED | hipabi.LAYOUT_BINS)
+    layouts = hipabi.ct.c_int()
+    ctx._ck(ctx.lib.so_ellpack_dims(dE.h, None, None, None, None, hipabi.ct.byref(layouts)))
+    assert layouts.value == hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS
+    dE.free()
+    assert np.array_equal(gpu_matmul(ctx, E, X, b, "relu", TILED), oracle.matmul(as_oracle(E), X, b, "relu"))
+    # a duplicated column is "not ascending" too
+    E2 = datagen.encode_dense(sparse_matrix(rng, 64, 300, .5))
+    E2.idx[5, 1] = E2.idx[5, 0]
+    assert np.array_equal(gpu_matmul(ctx, E2, X[:300], b[:64], "none", TILED), oracle.matmul(as_oracle(E2), X[:300], b[:64]))

@@ -212,6 +212,9 @@ def test_python_runtime_wrappers(oracle, tmp_path):
     bs = [rng.standard_normal(24).astype(np.float32), rng.standard_normal(8).astype(np.float32)]
     path = ow.save(str(tmp_path / "g.onnx"), ow.mlp_model(Ws, ["Relu", None], 4, bs, use_gemm=True))
     model = OnnxSparseModel(path)
+    # the reference's plan entries are (op, E, b, attrs) (python/sparse_onnx.py:27-32)
+    assert [op for op, E, b, attrs in model.layers] == ["matmul", "relu", "matmul"]
+    assert all(attrs == {} for op, E, b, attrs in model.layers) and model.layers[1][1] is None
     x = rng.standard_normal(16).astype(np.float32)
     y = model.run(x)                                          # 1-D input: matvec path
     ref = Ws[1].astype(np.float64) @ np.maximum(Ws[0].astype(np.float64) @ x + bs[0], 0) + bs[1]
@@ -326,3 +329,48 @@ def test_cpp_caller_of_the_reference_headers(oracle, tmp_path):
                        capture_output=True, text=True, timeout=100)
     assert r.returncode == 0, r.stdout + r.stderr
     assert r.stdout.count("ok  ") == 9 and "FAIL" not in r.stdout
+
+
+def _run_device(model, ctx, X_bm):
+    """X_bm (B, features...) -> (B, out features...) through SparseOnnxModel::run_device on HBM buffers
+    allocated through the C ABI."""
+    B = X_bm.shape[0]
+    Xf = np.ascontiguousarray(X_bm.reshape(B, -1).T)               # [features x B], the C++ contract
+    out_features = int(np.prod(model.output_shape()[1:]))
+    dX = ctx.array(Xf)
+    dY = ctx.array(np.full((out_features + 64, B), np.nan, np.float32))   # 64 guard rows behind the output
+    model.run_device(dX.ptr, B, dY.ptr)
+    got = dY.download()
+    dX.free()
+    dY.free()
+    assert np.isnan(got[out_features:]).all(), "run_device wrote past its [out_features x B] output"
+    return np.ascontiguousarray(got[:out_features].T).reshape([B] + list(model.output_shape()[1:]))
+
+
+def test_run_device_mlp_wide_hidden_layers(backend, ctx, oracle, tmp_path):
+    """run_device on a chain whose hidden tensors are wider than its output and share the output's
+    arena slot (slots are recycled after a tensor's last reader): the caller's [out x B] buffer
+    receives the last layer only, and the result has run()'s bits.  Batch 24 is not padded, 10 is
+    (no convolutions: never), so both run_device paths with an MLP and both with a CNN are taken."""
+    rng = np.random.default_rng(21)
+    dims, B = (60, 256, 256, 256, 10), 24
+    Ws = [datagen.magnitude_prune(rng.standard_normal((o, i)).astype(np.float32), .8) for i, o in zip(dims[:-1], dims[1:])]
+    acts = ["Relu", "Relu", "Relu", None]
+    model = backend.SparseOnnxModel(ow.save(str(tmp_path / "mlp.onnx"), ow.mlp_model(Ws, acts, B)))
+    X = rng.standard_normal((B, 60)).astype(np.float32)
+    Y = model.run(X)
+    assert np.array_equal(Y, oracle_mlp(oracle, Ws, acts, X))
+    assert np.array_equal(_run_device(model, ctx, X), Y)
+    assert np.array_equal(_run_device(model, ctx, X[:10]), Y[:10])     # another batch: resize, then run
+    assert np.array_equal(_run_device(model, ctx, X), Y)
+
+
+@pytest.mark.parametrize("B", [32, 5])
+def test_run_device_cnn(backend, ctx, tmp_path, B):
+    """run_device on a ResNet-shaped stack at a batch carried as is (32) and one carried padded (5)."""
+    payload, _ = datagen.resnet18_onnx(seed=5, batch=B, hw=32, sparsity=0.8, classes=10, width=16)
+    model = backend.SparseOnnxModel(ow.save(str(tmp_path / "r18.onnx"), payload))
+    X = np.random.default_rng(2).standard_normal((B, 3, 32, 32)).astype(np.float32)
+    Y = model.run(X)
+    assert np.array_equal(_run_device(model, ctx, X), Y)
+    assert np.array_equal(_run_device(model, ctx, X), Y)
