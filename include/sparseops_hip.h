@@ -200,6 +200,35 @@ so_status so_conv2d(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint
 so_status so_conv2d_add(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B,
                         const float *dBias, const float *dResidual, float *dY, int act);
 
+/* ---- row-block-merged (RBM) format ---------------------------------------
+ * RBMPlan / RBMBlock / RBMColPair (include/rbm_conv.hpp:8-27) as build_rbm_from_ellpack
+ * (src/layers/rbm_conv.cpp:7-73) produces them, flattened into five arrays: block b holds rows
+ * [b*Ct_max, min(M, (b+1)*Ct_max)) of the M x N matrix; its union columns (RBMBlock::krel) are
+ * krel[block_union[b] .. block_union[b+1]), ascending; union column u owns pairs colptr[u] ..
+ * colptr[u+1] (RBMBlock::colptr made absolute over all blocks), and pair p is (pair_row[p], pair_w[p])
+ * = RBMColPair{row inside the block, weight}, rows ascending.  The arrays are validated (SO_ERR_BOUNDS)
+ * and copied; the handle is what convolution plans build their kernel streams from.  Biases are not
+ * part of the handle: so_conv2d takes them per call, like the other kernels. */
+typedef struct so_rbm so_rbm;
+so_status so_rbm_upload(so_ctx *ctx, uint32_t M, uint32_t N, uint32_t Ct_max, uint32_t nblocks,
+                        const uint32_t *block_union, const uint32_t *krel, const uint32_t *colptr,
+                        const uint16_t *pair_row, const float *pair_w, so_rbm **out);
+so_status so_rbm_free(so_ctx *ctx, so_rbm *R);
+so_status so_rbm_dims(const so_rbm *R, uint32_t *M, uint32_t *N, uint32_t *Ct_max, uint32_t *nblocks,
+                      uint64_t *total_union, uint64_t *total_pairs);
+/* Attach the format to a convolution plan (ConvAttr::rbm / use_rbm, include/sparse_onnx.hpp:66-98;
+ * the reference builds it at load for Cout >= 32 and K >= 64, src/sparse_onnx.cpp:499-502): so_conv2d
+ * and so_conv2d_add then run conv2d_rbm_fmajor_implicit's algorithm (src/layers/conv_kernels.cpp:66-147)
+ * -- every union column's input operand fetched once and applied to all rows of the block that use
+ * it -- whenever the plan has its LDS-windowed layout and B is a multiple of 4, and the per-row
+ * kernels otherwise; the results have the same bits either way.  Blocks of at most 8 rows.  R must
+ * describe the plan's weights and outlive the plan; NULL detaches.  Not during graph capture. */
+so_status so_conv_plan_set_rbm(so_ctx *ctx, so_conv_plan *plan, const so_rbm *R);
+/* Inspection aid (no counterpart in the reference): out = {64-byte sets in the plan's streams,
+ * real (row, weight) pairs, slots the kernel multiplies through, slots per record}; zeros when
+ * the plan has no streams. */
+so_status so_conv_plan_rbm_info(const so_conv_plan *plan, uint64_t out[4]);
+
 /* applyMaxPool / applyGlobalAveragePool (src/layers/pool.cpp:28-101, 103-154)
  * on [C][H][W][B]; GAP writes [C][B]. */
 so_status so_maxpool(so_ctx *ctx, const so_pool_geom *p, const float *dX, uint32_t B, float *dY);

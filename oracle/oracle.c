@@ -18,6 +18,10 @@
  *   orc_act                 numpy maximum / 1/(1+exp(-x)) / tanh in fp64, compiled reference in-place kernels
  *   orc_conv2d_pf           7-loop brute force, torch conv2d, 1x1 == matmul, delta kernel == shift,
  *                           compiled reference conv2d_patchmajor_tiled (bit-exact up to the sign of zero)
+ *   orc_rbm_build           hand-written known answer, (column,row)-sorted numpy triples, decode(RBM) == W,
+ *                           compiled reference build_rbm_from_ellpack (identical arrays)
+ *   orc_conv2d_rbm_pf       orc_conv2d_pf (same bits: per-channel order is unchanged), compiled reference
+ *                           conv2d_rbm_fmajor_implicit, 1x1 == orc_matmul
  *   orc_maxpool_pf          numpy brute force, torch max_pool2d
  *   orc_gap_pf              numpy mean (tolerance), explicit (h,w)-ordered fp32 sum times reciprocal
  *   orc_add                 numpy
@@ -238,6 +242,106 @@ void orc_conv2d_pf(const float *Wd, const uint32_t *idx, const uint32_t *nnz, ui
                     for (uint32_t b = 0; b < B; ++b) yp[b] = fmaf(w, xp[b], yp[b]);
                 }
                 for (uint32_t b = 0; b < B; ++b) yp[b] = orc_act1(yp[b], act);
+            }
+}
+
+/* ------------------------------------------------ row-block-merged format */
+
+typedef struct { uint32_t k; uint32_t r; float w; } orc_trip;
+
+static int orc_trip_cmp(const void *a, const void *b)
+{
+    const orc_trip *x = (const orc_trip *)a, *y = (const orc_trip *)b;
+    if (x->k != y->k) return x->k < y->k ? -1 : 1;
+    return x->r < y->r ? -1 : (x->r > y->r ? 1 : 0);
+}
+
+/* build_rbm_from_ellpack (src/layers/rbm_conv.cpp:7-73), flattened: per block of Ct_max rows the
+ * (column, row in block, weight) triples of the rows' first nnz slots (:23-31) are ordered by
+ * (column, row) (:38-39) and cut into runs of equal column, one union column per run (:41-63).
+ * block_union[b] = union columns before block b; colptr is absolute over all blocks.  Called
+ * twice: with krel == NULL it only counts.  Returns via sizes = {union columns, pairs}. */
+void orc_rbm_build(const float *Wd, const uint32_t *idx, const uint32_t *nnz, uint32_t m, uint32_t r,
+                   uint32_t Ct_max, uint32_t *block_union, uint32_t *krel, uint32_t *colptr,
+                   uint16_t *pair_row, float *pair_w, uint64_t *sizes)
+{
+    orc_trip *all = (orc_trip *)malloc(sizeof(orc_trip) * ((size_t)Ct_max * r + 1));
+    uint64_t U = 0, P = 0;
+    uint32_t b = 0;
+    if (block_union) block_union[0] = 0;
+    if (krel) colptr[0] = 0;
+    for (uint32_t M0 = 0; M0 < m; M0 += Ct_max, ++b) {
+        const uint32_t Ct = m - M0 < Ct_max ? m - M0 : Ct_max;
+        size_t cnt = 0;
+        for (uint32_t rr = 0; rr < Ct; ++rr) {
+            const size_t base = (size_t)(M0 + rr) * r;
+            for (uint32_t j = 0; j < nnz[M0 + rr]; ++j) {
+                all[cnt].k = idx[base + j];
+                all[cnt].r = rr;
+                all[cnt].w = Wd[base + j];
+                ++cnt;
+            }
+        }
+        qsort(all, cnt, sizeof(orc_trip), orc_trip_cmp);
+        for (size_t t = 0; t < cnt; ++t) {
+            if (t == 0 || all[t].k != all[t - 1].k) {
+                if (krel) krel[U] = all[t].k;
+                ++U;
+            }
+            if (krel) {
+                pair_row[P] = (uint16_t)all[t].r;
+                pair_w[P] = all[t].w;
+                colptr[U] = (uint32_t)(P + 1);
+            }
+            ++P;
+        }
+        if (block_union) block_union[b + 1] = (uint32_t)U;
+    }
+    free(all);
+    sizes[0] = U;
+    sizes[1] = P;
+}
+
+/* conv2d_rbm_fmajor_implicit (src/layers/conv_kernels.cpp:66-147) on the [C][H][W][B] layout: per
+ * output pixel and block the accumulators start at the bias (:100-104); the block's union columns
+ * are walked once in order, a tap outside the image is skipped (:112-114), its input vector is
+ * multiply-added (fused) into every row that has a pair at that column (:118-123); optional ReLU
+ * (:126-130; the other activations are this build's epilogues).  Blocks of at most 64 rows. */
+void orc_conv2d_rbm_pf(const uint32_t *block_union, const uint32_t *krel, const uint32_t *colptr,
+                       const uint16_t *pair_row, const float *pair_w, uint32_t Ct_max,
+                       const orc_conv_geom *g, const float *X, uint32_t B,
+                       const float *bias, int act, float *Y)
+{
+    const uint32_t H = g->H_in, W = g->W_in, Ho = g->H_out, Wo = g->W_out;
+    const uint32_t kHW = g->kH * g->kW;
+    const uint32_t nblocks = (g->Cout + Ct_max - 1) / Ct_max;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (uint32_t ho = 0; ho < Ho; ++ho)
+        for (uint32_t wo = 0; wo < Wo; ++wo)
+            for (uint32_t blk = 0; blk < nblocks; ++blk) {
+                const uint32_t M0 = blk * Ct_max;
+                const uint32_t Ct = g->Cout - M0 < Ct_max ? g->Cout - M0 : Ct_max;
+                float *yp[64];
+                for (uint32_t rr = 0; rr < Ct; ++rr) {
+                    yp[rr] = Y + (((size_t)(M0 + rr) * Ho + ho) * Wo + wo) * B;
+                    const float b0 = bias ? bias[M0 + rr] : 0.0f;
+                    for (uint32_t b = 0; b < B; ++b) yp[rr][b] = b0;
+                }
+                for (uint32_t u = block_union[blk]; u < block_union[blk + 1]; ++u) {
+                    const uint32_t k = krel[u];
+                    const uint32_t cin = k / kHW, kh = (k / g->kW) % g->kH, kw = k % g->kW;
+                    const int32_t hin = (int32_t)(ho * g->stride_h) + (int32_t)(kh * g->dil_h) - (int32_t)g->pad_h;
+                    const int32_t win = (int32_t)(wo * g->stride_w) + (int32_t)(kw * g->dil_w) - (int32_t)g->pad_w;
+                    if ((uint32_t)hin >= H || (uint32_t)win >= W) continue;
+                    const float *xp = X + (((size_t)cin * H + (uint32_t)hin) * W + (uint32_t)win) * B;
+                    for (uint32_t p = colptr[u]; p < colptr[u + 1]; ++p) {
+                        float *y = yp[pair_row[p]];
+                        const float w = pair_w[p];
+                        for (uint32_t b = 0; b < B; ++b) y[b] = fmaf(w, xp[b], y[b]);
+                    }
+                }
+                for (uint32_t rr = 0; rr < Ct; ++rr)
+                    for (uint32_t b = 0; b < B; ++b) yp[rr][b] = orc_act1(yp[rr][b], act);
             }
 }
 

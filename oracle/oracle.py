@@ -80,6 +80,28 @@ class EllpackArrays:
         return int(self.nnz.sum(dtype=np.int64))
 
 
+class RbmArrays:
+    """build_rbm_from_ellpack's result (RBMPlan, include/rbm_conv.hpp:8-27) with the per-block vectors
+    laid end to end: block b = rows [b*Ct_max, ...) owns union columns krel[block_union[b] :
+    block_union[b+1]]; union column u owns pairs colptr[u] : colptr[u+1] (colptr made absolute over
+    all blocks), pair p = (pair_row[p], pair_w[p])."""
+
+    def __init__(self, M, N, Ct_max, block_union, krel, colptr, pair_row, pair_w):
+        self.M, self.N, self.Ct_max = int(M), int(N), int(Ct_max)
+        self.block_union = np.ascontiguousarray(block_union, dtype=np.uint32)
+        self.krel = np.ascontiguousarray(krel, dtype=np.uint32)
+        self.colptr = np.ascontiguousarray(colptr, dtype=np.uint32)
+        self.pair_row = np.ascontiguousarray(pair_row, dtype=np.uint16)
+        self.pair_w = np.ascontiguousarray(pair_w, dtype=np.float32)
+        self.nblocks = len(self.block_union) - 1
+
+    def same_as(self, o):
+        return ((self.M, self.N, self.Ct_max) == (o.M, o.N, o.Ct_max) and
+                all(np.array_equal(getattr(self, k), getattr(o, k))
+                    for k in ("block_union", "krel", "colptr", "pair_row")) and
+                np.array_equal(self.pair_w.view(np.uint32), o.pair_w.view(np.uint32)))
+
+
 class Oracle:
     def __init__(self, path=None):
         path = path or os.path.join(_HERE, "liboracle.so")
@@ -97,6 +119,11 @@ class Oracle:
         L.orc_matvec.argtypes = [_f32p, _u32p, _u32p, ct.c_uint32, ct.c_uint32, ct.c_uint32, _f32p, _f32p, _f32p]
         L.orc_conv2d_pf.argtypes = [_f32p, _u32p, _u32p, ct.c_uint32, ct.POINTER(ConvGeom), _f32p,
                                     ct.c_uint32, _f32p, ct.c_int, _f32p]
+        _u16p = ct.POINTER(ct.c_uint16)
+        L.orc_rbm_build.argtypes = [_f32p, _u32p, _u32p, ct.c_uint32, ct.c_uint32, ct.c_uint32, _u32p, _u32p, _u32p,
+                                    _u16p, _f32p, ct.POINTER(ct.c_uint64)]
+        L.orc_conv2d_rbm_pf.argtypes = [_u32p, _u32p, _u32p, _u16p, _f32p, ct.c_uint32, ct.POINTER(ConvGeom), _f32p,
+                                        ct.c_uint32, _f32p, ct.c_int, _f32p]
         L.orc_maxpool_pf.argtypes = [ct.POINTER(PoolGeom), _f32p, ct.c_uint32, _f32p]
         L.orc_gap_pf.argtypes = [ct.c_uint32, ct.c_uint32, ct.c_uint32, _f32p, ct.c_uint32, _f32p]
         L.orc_add.argtypes = [_f32p, _f32p, ct.c_size_t, _f32p]
@@ -150,6 +177,30 @@ class Oracle:
         Y = np.empty((g.Cout, g.H_out, g.W_out, B), dtype=np.float32)
         self.lib.orc_conv2d_pf(_fp(E.Wd), _up(E.idx), _up(E.nnz), E.r, ct.byref(g), _fp(X), B,
                                _fp(bias), ACT[act], _fp(Y))
+        return Y
+
+    def rbm_build(self, E, Ct_max=8):
+        """build_rbm_from_ellpack restated (orc_rbm_build) -> RbmArrays."""
+        nb = (E.m + Ct_max - 1) // Ct_max
+        sizes = (ct.c_uint64 * 2)()
+        bu = np.zeros(nb + 1, dtype=np.uint32)
+        self.lib.orc_rbm_build(_fp(E.Wd), _up(E.idx), _up(E.nnz), E.m, E.r, Ct_max, _up(bu), None, None, None, None, sizes)
+        U, P = int(sizes[0]), int(sizes[1])
+        krel, colptr = np.zeros(U, np.uint32), np.zeros(U + 1, np.uint32)
+        prow, pw = np.zeros(P, np.uint16), np.zeros(P, np.float32)
+        self.lib.orc_rbm_build(_fp(E.Wd), _up(E.idx), _up(E.nnz), E.m, E.r, Ct_max, _up(bu), _up(krel), _up(colptr),
+                               prow.ctypes.data_as(ct.POINTER(ct.c_uint16)), _fp(pw), sizes)
+        return RbmArrays(E.m, E.n, Ct_max, bu, krel, colptr, prow, pw)
+
+    def conv2d_rbm_pf(self, R, g, X, B, bias=None, act="none"):
+        """conv2d_rbm_fmajor_implicit restated on [C][H][W][B] (orc_conv2d_rbm_pf)."""
+        assert R.Ct_max <= 64
+        X = _f32(X)
+        bias = None if bias is None else _f32(bias)
+        Y = np.empty((g.Cout, g.H_out, g.W_out, B), dtype=np.float32)
+        self.lib.orc_conv2d_rbm_pf(_up(R.block_union), _up(R.krel), _up(R.colptr),
+                                   R.pair_row.ctypes.data_as(ct.POINTER(ct.c_uint16)), _fp(R.pair_w), R.Ct_max,
+                                   ct.byref(g), _fp(X), B, _fp(bias), ACT[act], _fp(Y))
         return Y
 
     def maxpool_pf(self, X, C, H, W, B, k, s, pad):
@@ -208,6 +259,8 @@ class Ref:
         for nm in ("ref_relu_inplace", "ref_sigmoid_inplace", "ref_tanh_inplace"):
             getattr(L, nm).argtypes = [_f32p, ct.c_size_t]
         L.ref_conv.argtypes = [_f32p, _u32p, _f32p, ct.c_int, ct.c_int, _f32p, ct.c_uint32, _f32p]
+        L.ref_rbm_sizes.argtypes = [ct.c_void_p, ct.c_uint32, _u32p]
+        L.ref_rbm_copy.argtypes = [ct.c_void_p, ct.c_uint32, _u32p, _u32p, _u32p, ct.POINTER(ct.c_uint16), _f32p]
 
     class Handle:
         def __init__(self, lib, h):
@@ -265,6 +318,16 @@ class Ref:
         y = _f32(x).copy()
         getattr(self.lib, "ref_%s_inplace" % act)(_fp(y), y.size)
         return y
+
+    def rbm_build(self, h, Ct_max=8):
+        """The reference's own build_rbm_from_ellpack on the handle's matrix -> RbmArrays."""
+        sizes = np.zeros(3, dtype=np.uint32)
+        self.lib.ref_rbm_sizes(h.h, Ct_max, _up(sizes))
+        nb, U, P = (int(v) for v in sizes)
+        bu, krel, colptr = np.zeros(nb + 1, np.uint32), np.zeros(U, np.uint32), np.zeros(U + 1, np.uint32)
+        prow, pw = np.zeros(P, np.uint16), np.zeros(P, np.float32)
+        self.lib.ref_rbm_copy(h.h, Ct_max, _up(bu), _up(krel), _up(colptr), prow.ctypes.data_as(ct.POINTER(ct.c_uint16)), _fp(pw))
+        return RbmArrays(h.m, h.n, Ct_max, bu, krel, colptr, prow, pw)
 
     def conv(self, Wdense, g, src, B, bias=None, fuse_relu=False, variant=0):
         Wdense, src = _f32(Wdense), _f32(src)

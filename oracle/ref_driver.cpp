@@ -140,4 +140,33 @@ void ref_conv(const float *Wdense, const uint32_t *geom, const float *bias, int 
     }
 }
 
+// build_rbm_from_ellpack on the handle's matrix, flattened: sizes = {blocks, union columns, pairs};
+// block_union[b] = union columns before block b, colptr made absolute over all blocks.
+void ref_rbm_sizes(void *h, uint32_t Ct_max, uint32_t *sizes)
+{
+    const RBMPlan P = build_rbm_from_ellpack(*static_cast<Ellpack *>(h), nullptr, Ct_max);
+    sizes[0] = uint32_t(P.blocks.size());
+    sizes[1] = sizes[2] = 0;
+    for (const RBMBlock &b : P.blocks) { sizes[1] += uint32_t(b.krel.size()); sizes[2] += uint32_t(b.pairs.size()); }
+}
+
+void ref_rbm_copy(void *h, uint32_t Ct_max, uint32_t *block_union, uint32_t *krel, uint32_t *colptr,
+                  uint16_t *pair_row, float *pair_w)
+{
+    const RBMPlan P = build_rbm_from_ellpack(*static_cast<Ellpack *>(h), nullptr, Ct_max);
+    uint32_t u = 0, p = 0;
+    block_union[0] = 0;
+    colptr[0] = 0;
+    for (size_t b = 0; b < P.blocks.size(); ++b) {
+        const RBMBlock &B = P.blocks[b];
+        for (size_t k = 0; k < B.krel.size(); ++k) {
+            krel[u] = B.krel[k];
+            colptr[u + 1] = p + B.colptr[k + 1];
+            ++u;
+        }
+        for (const RBMColPair &q : B.pairs) { pair_row[p] = q.row; pair_w[p] = q.w; ++p; }
+        block_union[b + 1] = u;
+    }
+}
+
 } // extern "C"

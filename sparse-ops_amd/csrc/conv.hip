@@ -15,6 +15,7 @@
 // the CU's L1.  Accumulation is bias first, then one fused multiply-add per stored
 // nonzero in ascending slot order, as in the reference.
 #include "so_internal.h"
+#include "conv_internal.h"
 #include "dpp_steps.h"
 
 #include <algorithm>
@@ -22,35 +23,6 @@
 #include <cstring>
 #include <new>
 #include <vector>
-
-// What the LDS-windowed kernel needs on top of the plan; built only for geometries it suits.
-// The input channels are cut into chunks of `cc`; for one chunk and one tile of TH x TW output
-// pixels the input window is IH x IW pixels.  A stored nonzero becomes the entry {weight bits,
-// pixel offset of its tap inside the chunk's window}.  Output channels are taken `cpw` at a
-// time (the channels one wave accumulates); the entries of such a channel group are one
-// contiguous stream in the order the wave consumes them: chunk by chunk, inside a chunk channel
-// by channel, inside a channel in slot order (slots are ordered by input channel, so a chunk is
-// a slot range).  Every (chunk, channel) run is padded to a multiple of four entries with
-// {-0.0, offset of an all-zero plane kept behind the window}: fma(-0, +0, acc) leaves any
-// accumulator as it is.
-struct so_conv_window {
-    uint32_t TH = 0, TW = 0, IH = 0, IW = 0, cc = 0, nch = 0, tiles_x = 0, tiles_y = 0;
-    uint32_t groups = 0;          // ceil(Cout / cpw)
-    int cpw = 0;                  // output channels per wave
-    uint32_t lpp = 0;             // lanes per pixel (batch tile / 4) the chunk size was chosen for: 4, 2 or 1
-    int2 *d_stream = nullptr;     // all groups' streams, followed by one padding quad
-    uint32_t *d_gbase = nullptr;  // [groups]: first quad (4 entries) of the group's stream
-    uint32_t *d_quads = nullptr;  // [groups * nch * cpw]: quads of (group, chunk, channel in group)
-};
-
-struct so_conv_plan {
-    uint32_t tuned_batch = 32;   // batch the windowed layout was sized for
-    uint32_t tried_lpp = 0;      // lanes per pixel of the last attempt to build the windowed layout
-    so_conv_geom g;
-    const so_ellpack *E = nullptr;
-    int2 *d_taps = nullptr;  // per slot: x = (cin*H + dh)*W + dw (elements of B floats), y = dh<<16 | (dw & 0xffff)
-    so_conv_window win;      // win.cc == 0: not built
-};
 
 namespace {
 
@@ -266,29 +238,6 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
 // multiply-adds run in slot order (chunks ascend, slots ascend inside a chunk): same bits as
 // the kernel above.  Windows are double-buffered: chunk t+1 is fetched into registers while
 // chunk t is computed.
-constexpr int kWinThreads = 1024;
-constexpr int kWinMaxPerThread = 6;   // float4 window elements a thread copies per chunk
-constexpr uint32_t kWinLPP = 4;       // lanes per pixel of the preferred batch tile ...
-constexpr uint32_t kWinBT = 4 * kWinLPP;   // ... of 16; batches that are only multiples of 8 or 4 use tiles of 8 or 4
-
-// Lanes per pixel for batch B: the largest batch tile (16, 8, 4) that divides B; 0 if none does.
-inline uint32_t window_lpp(uint32_t B) { return B % 16 == 0 ? 4u : B % 8 == 0 ? 2u : B % 4 == 0 ? 1u : 0u; }
-
-struct WinArgs {
-    uint32_t TH, TW, IH, IW, cc, nch, tiles_x, pg, cg, groups;
-    uint32_t win_f4;    // float4 elements of one chunk's window
-    uint32_t buf_f4;    // window plus the zero plane: stride between the two buffers
-    uint32_t nbuf;      // 2: double-buffered windows; 1: a single chunk, nothing to overlap
-    uint32_t sth, stw;  // window pixels between neighbouring output pixels
-    uint32_t sbh, sbw;  // input pixels between neighbouring window pixels
-};
-
-// Along an axis on which the kernel has a single tap, a strided convolution reads only every
-// stride-th input pixel: the window then holds just those (one window pixel per output pixel)
-// instead of all the pixels in between.
-inline uint32_t window_step(uint32_t k, uint32_t stride) { return k == 1 ? 1u : stride; }
-inline uint32_t window_subsample(uint32_t k, uint32_t stride) { return k == 1 ? stride : 1u; }
-
 template <int CPW, int LPP, int ACT>
 __global__ __launch_bounds__(kWinThreads)
 void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__restrict__ gbase,
@@ -814,6 +763,7 @@ extern "C" so_status so_conv_plan_free(so_ctx *ctx, so_conv_plan *plan)
     if (ctx && ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (plan->d_taps) (void)hipFree(plan->d_taps);
     free_window(plan);
+    so_conv_rbm_release(plan);
     delete plan;
     return SO_OK;
 }
@@ -846,7 +796,9 @@ extern "C" so_status so_conv_plan_tune(so_ctx *ctx, so_conv_plan *plan, uint32_t
     SO_HIP(hipStreamSynchronize(ctx->stream));      // no launch may still be reading the old arrays
     free_window(plan);
     plan->tuned_batch = batch;
-    return build_window(ctx, plan, idx, nnz, Wd, batch);
+    s = build_window(ctx, plan, idx, nnz, Wd, batch);
+    if (s != SO_OK) return s;
+    return so_conv_rbm_rebuild(ctx, plan);          // the record streams follow the window's chunks
 }
 
 extern "C" so_status so_conv_plan_window(const so_conv_plan *plan, uint32_t out[8])
@@ -876,6 +828,16 @@ static so_status conv2d_dispatch(so_ctx *ctx, const so_conv_plan *plan, const fl
     // 16, 8 or 4 (SPARSEOPS_CONV_WINDOW=1 forces it whenever possible, =0 forbids it: tuning and tests).
     const uint32_t lpp = window_lpp(B);
     if (plan->win.cc != 0 && lpp != 0 && (align & 15) == 0 && (uint64_t)plan->win.cc * g.H_in * g.W_in * B < (1ull << 31)) {
+        // a plan that carries the row-block-merged streams runs that kernel (SPARSEOPS_CONV_RBM=0 forbids it)
+        if (plan->rbm.d_sets && ctx->tune.conv_rbm != 0) {
+            bool done = false;
+            const so_status s = so_conv_rbm_launch(ctx, plan, dX, B, dBias, dResid, dY, act, ctx->tune.conv_rbm == 1, &done);
+            if (s != SO_OK) return s;
+            if (done) {
+                SO_LAUNCH_CHECK();
+                return SO_OK;
+            }
+        }
         const bool forced = ctx->tune.conv_window == 1;
         if (ctx->tune.conv_window != 0) {
             bool done = false;

@@ -1,0 +1,74 @@
+// Definitions shared by the convolution translation units (conv.hip, conv_rbm.hip).
+#pragma once
+
+#include "so_internal.h"
+
+// What the LDS-windowed kernel needs on top of the plan; built only for geometries it suits.
+// The input channels are cut into chunks of `cc`; for one chunk and one tile of TH x TW output
+// pixels the input window is IH x IW pixels.  A stored nonzero becomes the entry {weight bits,
+// pixel offset of its tap inside the chunk's window}.  Output channels are taken `cpw` at a
+// time (the channels one wave accumulates); the entries of such a channel group are one
+// contiguous stream in the order the wave consumes them: chunk by chunk, inside a chunk channel
+// by channel, inside a channel in slot order (slots are ordered by input channel, so a chunk is
+// a slot range).  Every (chunk, channel) run is padded to a multiple of four entries with
+// {-0.0, offset of an all-zero plane kept behind the window}: fma(-0, +0, acc) leaves any
+// accumulator as it is.
+struct so_conv_window {
+    uint32_t TH = 0, TW = 0, IH = 0, IW = 0, cc = 0, nch = 0, tiles_x = 0, tiles_y = 0;
+    uint32_t groups = 0;          // ceil(Cout / cpw)
+    int cpw = 0;                  // output channels per wave
+    uint32_t lpp = 0;             // lanes per pixel (batch tile / 4) the chunk size was chosen for: 4, 2 or 1
+    int2 *d_stream = nullptr;     // all groups' streams, followed by one padding quad
+    uint32_t *d_gbase = nullptr;  // [groups]: first quad (4 entries) of the group's stream
+    uint32_t *d_quads = nullptr;  // [groups * nch * cpw]: quads of (group, chunk, channel in group)
+};
+
+// Record streams of the row-block-merged kernel (conv_rbm.hip) for the plan's current window layout.
+struct so_conv_rbm {
+    const so_rbm *src = nullptr;     // the attached format; must outlive the plan
+    void *d_sets = nullptr;          // 64-byte sets of two records, all blocks, chunk after chunk
+    uint32_t *d_gbase = nullptr;     // [blocks]: first set of the block's stream
+    uint32_t *d_counts = nullptr;    // [blocks * chunks]: sets the loop walks for (block, chunk); 0: none
+    uint64_t total_sets = 0, real_pairs = 0, slots = 0;
+};
+
+struct so_conv_plan {
+    uint32_t tuned_batch = 32;   // batch the windowed layout was sized for
+    uint32_t tried_lpp = 0;      // lanes per pixel of the last attempt to build the windowed layout
+    so_conv_geom g;
+    const so_ellpack *E = nullptr;
+    int2 *d_taps = nullptr;  // per slot: x = (cin*H + dh)*W + dw (elements of B floats), y = dh<<16 | (dw & 0xffff)
+    so_conv_window win;      // win.cc == 0: not built
+    so_conv_rbm rbm;         // rbm.d_sets == nullptr: no streams
+};
+
+// conv_rbm.hip
+void so_conv_rbm_release(so_conv_plan *plan);
+so_status so_conv_rbm_rebuild(so_ctx *ctx, so_conv_plan *plan);
+so_status so_conv_rbm_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, uint32_t B, const float *dBias,
+                             const float *dResid, float *dY, int act, bool forced, bool *done);
+
+
+constexpr int kWinThreads = 1024;
+constexpr int kWinMaxPerThread = 6;   // float4 window elements a thread copies per chunk
+constexpr uint32_t kWinLPP = 4;       // lanes per pixel of the preferred batch tile ...
+constexpr uint32_t kWinBT = 4 * kWinLPP;   // ... of 16; batches that are only multiples of 8 or 4 use tiles of 8 or 4
+
+// Lanes per pixel for batch B: the largest batch tile (16, 8, 4) that divides B; 0 if none does.
+inline uint32_t window_lpp(uint32_t B) { return B % 16 == 0 ? 4u : B % 8 == 0 ? 2u : B % 4 == 0 ? 1u : 0u; }
+
+struct WinArgs {
+    uint32_t TH, TW, IH, IW, cc, nch, tiles_x, pg, cg, groups;
+    uint32_t win_f4;    // float4 elements of one chunk's window
+    uint32_t buf_f4;    // window plus the zero plane: stride between the two buffers
+    uint32_t nbuf;      // 2: double-buffered windows; 1: a single chunk, nothing to overlap
+    uint32_t sth, stw;  // window pixels between neighbouring output pixels
+    uint32_t sbh, sbw;  // input pixels between neighbouring window pixels
+};
+
+// Along an axis on which the kernel has a single tap, a strided convolution reads only every
+// stride-th input pixel: the window then holds just those (one window pixel per output pixel)
+// instead of all the pixels in between.
+inline uint32_t window_step(uint32_t k, uint32_t stride) { return k == 1 ? 1u : stride; }
+inline uint32_t window_subsample(uint32_t k, uint32_t stride) { return k == 1 ? stride : 1u; }
+

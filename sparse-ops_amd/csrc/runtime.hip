@@ -64,6 +64,7 @@ static void read_tuning(so_tuning &t)
     t.conv_cpw = env_int("SPARSEOPS_CONV_CPW", 0);
     t.conv_tilepx = env_int("SPARSEOPS_CONV_TILEPX", 0);
     t.conv_vec = env_int("SPARSEOPS_CONV_VEC", 0);
+    t.conv_rbm = env_int("SPARSEOPS_CONV_RBM", -1);
 }
 
 extern "C" so_status so_tuning_reload(so_ctx *ctx)

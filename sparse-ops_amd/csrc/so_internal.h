@@ -20,6 +20,7 @@ struct so_tuning {
     int conv_cpw = 0;        // SPARSEOPS_CONV_CPW: most output channels per wave
     int conv_tilepx = 0;     // SPARSEOPS_CONV_TILEPX: most output pixels per tile
     int conv_vec = 0;        // SPARSEOPS_CONV_VEC: most batch entries per lane in the gather kernel
+    int conv_rbm = -1;       // SPARSEOPS_CONV_RBM: 0 forbids the row-block-merged kernel on plans that carry its streams
 };
 
 struct so_ctx {
@@ -78,6 +79,18 @@ struct so_ellpack {
     uint32_t *d_idxT = nullptr;
     so_bin bins[3];              // SO_LAYOUT_BINS
     so_tiled tiled;              // SO_LAYOUT_TILED
+};
+
+// Row-block-merged re-encoding of a matrix (include/rbm_conv.hpp:8-27 of the reference), flattened:
+// block b holds rows [b*Ct_max, min(M, (b+1)*Ct_max)); its union columns are krel[block_union[b] ..
+// block_union[b+1]) in ascending order; union column u owns the pairs colptr[u] .. colptr[u+1], each
+// a (row inside the block, weight), rows ascending.  Kept on the host: convolution plans turn it
+// into the record streams their kernel reads.
+struct so_rbm {
+    uint32_t M = 0, N = 0, Ct_max = 0, nblocks = 0;
+    std::vector<uint32_t> block_union, krel, colptr;
+    std::vector<uint16_t> pair_row;
+    std::vector<float> pair_w;
 };
 
 struct so_graph {

@@ -12,6 +12,7 @@
 #include "sparseops_hip.h"
 
 struct Ellpack;
+struct RBMPlan;
 
 namespace sparseops {
 
@@ -57,6 +58,11 @@ struct EllpackMirror {
 /// Upload E once (or again if `layouts` asks for more than is resident) and
 /// return the device handle.
 const so_ellpack *mirror(const Ellpack &E, int layouts);
+
+/// The row-block-merged plan handed to the device library (so_rbm_upload): its per-block vectors
+/// laid end to end.  The caller owns the handle (so_rbm_free).  Biases stay with the caller: the
+/// kernels take them per call.
+so_rbm *upload_rbm(const RBMPlan &plan);
 
 /// Device layouts to keep for Y = E * X with C dense columns (ROW, plus TILED
 /// where the LDS-staged kernel pays).

@@ -22,7 +22,7 @@ SYMBOLS = (
     "so_d2d so_fill_zero so_sync so_timer_begin so_timer_end so_ellpack_upload so_ellpack_free "
     "so_ellpack_dims so_ellpack_download so_ellpack_decode so_ellpack_encode so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
     "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_copy_rows so_graph_begin so_graph_end "
-    "so_graph_launch so_graph_free").split()
+    "so_graph_launch so_graph_free so_rbm_upload so_rbm_free so_rbm_dims so_conv_plan_set_rbm so_conv_plan_rbm_info").split()
 
 _vp = ct.c_void_p
 _u32 = ct.c_uint32
@@ -97,6 +97,12 @@ def load_library(path=None):
         "so_graph_end": [_vp, ct.POINTER(_vp)],
         "so_graph_launch": [_vp, _vp],
         "so_graph_free": [_vp, _vp],
+        "so_rbm_upload": [_vp, _u32, _u32, _u32, _u32, _vp, _vp, _vp, _vp, _vp, ct.POINTER(_vp)],
+        "so_rbm_free": [_vp, _vp],
+        "so_rbm_dims": [_vp, ct.POINTER(_u32), ct.POINTER(_u32), ct.POINTER(_u32), ct.POINTER(_u32),
+                        ct.POINTER(ct.c_uint64), ct.POINTER(ct.c_uint64)],
+        "so_conv_plan_set_rbm": [_vp, _vp, _vp],
+        "so_conv_plan_rbm_info": [_vp, ct.POINTER(ct.c_uint64)],
     }
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
@@ -267,6 +273,36 @@ class Context:
         self._ck(self.lib.so_conv_plan_window(plan, out))
         keys = ("tile_h", "tile_w", "window_h", "window_w", "chunk_channels", "chunks", "channels_per_wave")
         return dict(zip(keys, out[:7])) if out[4] else None
+
+    def upload_rbm(self, M, N, Ct_max, block_union, krel, colptr, pair_row, pair_w):
+        """The flattened row-block-merged format (see so_rbm_upload) -> handle."""
+        bu = np.ascontiguousarray(block_union, dtype=np.uint32)
+        krel = np.ascontiguousarray(krel, dtype=np.uint32)
+        colptr = np.ascontiguousarray(colptr, dtype=np.uint32)
+        prow = np.ascontiguousarray(pair_row, dtype=np.uint16)
+        pw = np.ascontiguousarray(pair_w, dtype=np.float32)
+        h = _vp()
+        self._ck(self.lib.so_rbm_upload(self.h, M, N, Ct_max, len(bu) - 1, _ptr(bu), _ptr(krel), _ptr(colptr),
+                                        _ptr(prow), _ptr(pw), ct.byref(h)))
+        return h.value
+
+    def rbm_dims(self, rbm):
+        M, N, Ct, nb = _u32(), _u32(), _u32(), _u32()
+        U, P = ct.c_uint64(), ct.c_uint64()
+        self._ck(self.lib.so_rbm_dims(rbm, ct.byref(M), ct.byref(N), ct.byref(Ct), ct.byref(nb), ct.byref(U), ct.byref(P)))
+        return dict(M=M.value, N=N.value, Ct_max=Ct.value, nblocks=nb.value, union=U.value, pairs=P.value)
+
+    def rbm_free(self, rbm):
+        self.lib.so_rbm_free(self.h, rbm)
+
+    def conv_plan_set_rbm(self, plan, rbm):
+        self._ck(self.lib.so_conv_plan_set_rbm(self.h, plan, rbm))
+
+    def conv_plan_rbm_info(self, plan):
+        """-> dict(sets, pairs, slots, slots_per_record) of the plan's RBM streams, or None without streams."""
+        out = (ct.c_uint64 * 4)()
+        self._ck(self.lib.so_conv_plan_rbm_info(plan, out))
+        return dict(sets=out[0], pairs=out[1], slots=out[2], slots_per_record=out[3]) if out[0] else None
 
     def conv_plan_free(self, plan):
         self.lib.so_conv_plan_free(self.h, plan)

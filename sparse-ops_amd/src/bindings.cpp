@@ -13,6 +13,7 @@
 #include "ellpack_matmul.hpp"
 #include "ellpack_matvec.hpp"
 #include "onnx_wire.hpp"
+#include "rbm_conv.hpp"
 #include "sparse_onnx.hpp"
 
 namespace py = pybind11;
@@ -158,6 +159,38 @@ PYBIND11_MODULE(sparseops_backend, mod)
         out["outputs"] = vis(m.graph.output);
         return out;
     });
+
+    // The row-block-merged plan (include/rbm_conv.hpp of the reference; not bound there).
+    py::class_<RBMBlock>(mod, "RBMBlock")
+        .def_readonly("M0", &RBMBlock::M0)
+        .def_readonly("Ct", &RBMBlock::Ct)
+        .def_property_readonly("krel", [](const RBMBlock &b) { return py::array_t<uint32_t>(py::ssize_t(b.krel.size()), b.krel.data()); })
+        .def_property_readonly("colptr", [](const RBMBlock &b) { return py::array_t<uint32_t>(py::ssize_t(b.colptr.size()), b.colptr.data()); })
+        .def_property_readonly("pair_row", [](const RBMBlock &b) {
+            py::array_t<uint16_t> out(py::ssize_t(b.pairs.size()));
+            for (std::size_t i = 0; i < b.pairs.size(); ++i) out.mutable_data()[i] = b.pairs[i].row;
+            return out;
+        })
+        .def_property_readonly("pair_w", [](const RBMBlock &b) {
+            py::array_t<float> out(py::ssize_t(b.pairs.size()));
+            for (std::size_t i = 0; i < b.pairs.size(); ++i) out.mutable_data()[i] = b.pairs[i].w;
+            return out;
+        })
+        .def_property_readonly("bias", [](const RBMBlock &b) { return py::array_t<float>(py::ssize_t(b.bias.size()), b.bias.data()); });
+    py::class_<RBMPlan>(mod, "RBMPlan")
+        .def_readonly("M", &RBMPlan::M)
+        .def_readonly("N", &RBMPlan::N)
+        .def_readonly("Ct_max", &RBMPlan::Ct_max)
+        .def_property_readonly("blocks", [](const RBMPlan &p) { return p.blocks; });
+    mod.def("build_rbm_from_ellpack", [](const Ellpack &E, const py::object &bias, uint32_t Ct_max) {
+        farray holder;
+        return build_rbm_from_ellpack(E, optional_bias(bias, holder, E.m), Ct_max);
+    }, py::arg("E"), py::arg("bias") = py::none(), py::arg("Ct_max") = 8,
+       "Row-block-merged re-encoding of an ELLPACK matrix (blocks of Ct_max rows, union columns, (row, weight) pairs)");
+
+    mod.def("reload_tuning", []() { sparseops::check(so_tuning_reload(sparseops::context()), "so_tuning_reload"); },
+            "Read the SPARSEOPS_* tuning overrides from the environment again (they are read when the process-wide "
+            "context is created); models pick the change up at their next resize_buffers");
 
     py::class_<SparseOnnxModel>(mod, "SparseOnnxModel")
         .def(py::init<const std::string &>(), "Load an ONNX model and pre-encode weights to ELLPACK")

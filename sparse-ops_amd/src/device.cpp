@@ -2,8 +2,10 @@
 #include "device.hpp"
 
 #include <new>
+#include <vector>
 
 #include "ellpack_encoder.hpp"
+#include "rbm_conv.hpp"
 
 namespace sparseops {
 
@@ -90,6 +92,28 @@ const so_ellpack *mirror(const Ellpack &E, int layouts)
     mir->layouts = layouts;
     E.device = std::move(mir);
     return E.device->handle;
+}
+
+so_rbm *upload_rbm(const RBMPlan &plan)
+{
+    std::vector<uint32_t> block_union{0}, krel, colptr{0};
+    std::vector<uint16_t> pair_row;
+    std::vector<float> pair_w;
+    for (const RBMBlock &b : plan.blocks) {
+        const uint32_t base = uint32_t(pair_w.size());
+        krel.insert(krel.end(), b.krel.begin(), b.krel.end());
+        for (std::size_t u = 1; u < b.colptr.size(); ++u) colptr.push_back(base + b.colptr[u]);
+        for (const RBMColPair &q : b.pairs) {
+            pair_row.push_back(q.row);
+            pair_w.push_back(q.w);
+        }
+        block_union.push_back(uint32_t(krel.size()));
+    }
+    so_rbm *handle = nullptr;
+    check(so_rbm_upload(context(), plan.M, plan.N, plan.Ct_max, uint32_t(plan.blocks.size()), block_union.data(), krel.data(),
+                        colptr.data(), pair_row.data(), pair_w.data(), &handle),
+          "so_rbm_upload");
+    return handle;
 }
 
 } // namespace sparseops

@@ -27,6 +27,7 @@ struct LayerPlan {
     Ellpack *E = nullptr;       // owned by Impl::weights
     const so_ellpack *dE = nullptr;
     so_conv_plan *conv = nullptr;
+    so_rbm *rbm = nullptr;      // Conv: the row-block-merged plan attached to `conv`, when one was built
     so_conv_geom cg{};
     std::vector<float> bias;    // host copy; device copy lives in Impl::bias_pool
     std::size_t bias_offset = 0;

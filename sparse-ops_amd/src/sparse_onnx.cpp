@@ -10,6 +10,7 @@
 #include <unordered_set>
 
 #include "model_impl.hpp"
+#include "rbm_conv.hpp"
 #include "onnx_wire.hpp"
 
 using namespace sparseops;
@@ -73,8 +74,10 @@ SparseOnnxModel::Impl::~Impl()
     so_ctx *ctx = nullptr;
     try { ctx = context(); } catch (...) { return; }
     if (graph) so_graph_free(ctx, graph);
-    for (auto &L : layers)
+    for (auto &L : layers) {
         if (L.conv) so_conv_plan_free(ctx, L.conv);
+        if (L.rbm) so_rbm_free(ctx, L.rbm);
+    }
 }
 
 SparseOnnxModel::~SparseOnnxModel() = default;
@@ -456,8 +459,17 @@ SparseOnnxModel::SparseOnnxModel(const std::string &onnx_path) : impl_(new Impl(
     for (auto &p : pend) {
         if (p.plan.op != Op::MatMul && p.plan.op != Op::Conv) continue;
         p.plan.dE = mirror(*p.plan.E, p.plan.op == Op::MatMul ? matmul_layouts(*p.plan.E, uint32_t(B0)) : SO_LAYOUT_ROW);
-        if (p.plan.op == Op::Conv)
+        if (p.plan.op == Op::Conv) {
             check(so_conv_plan_create(ctx, p.plan.dE, &p.plan.cg, &p.plan.conv), "so_conv_plan_create");
+            // The reference builds its row-block-merged plan for wide convolutions at load
+            // (src/sparse_onnx.cpp:499-502: Cout >= 32 and K >= 64, blocks of 8 channels) and never
+            // runs it; here the plan goes to the device library, whose so_conv2d walks it wherever
+            // that is the faster kernel for the batch at hand.
+            if (p.plan.cg.Cout >= 32 && p.plan.E->n >= 64) {
+                p.plan.rbm = upload_rbm(build_rbm_from_ellpack(*p.plan.E, nullptr, 8));
+                check(so_conv_plan_set_rbm(ctx, p.plan.conv, p.plan.rbm), "so_conv_plan_set_rbm");
+            }
+        }
         if (p.plan.has_bias) {
             p.plan.bias_offset = bias_total;
             bias_total += (p.plan.bias.size() + 63) / 64 * 64;

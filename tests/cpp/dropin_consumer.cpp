@@ -8,6 +8,7 @@
 #include "ellpack_encoder.hpp"
 #include "ellpack_matmul.hpp"
 #include "ellpack_matvec.hpp"
+#include "rbm_conv.hpp"
 #include "sparse_onnx.hpp"
 
 #include <cmath>
@@ -90,6 +91,29 @@ int main(int argc, char **argv)
         scale = std::max(scale, std::fabs(acc));
     }
     check(worst <= 1e-5 * scale, "ellpack_matvec within 1e-5 of the fp64 product");
+
+    // build_rbm_from_ellpack as the reference declares it (include/rbm_conv.hpp:31): every stored nonzero
+    // appears once, under its column, in a block's union list; columns and rows ascend
+    {
+        const RBMPlan plan = build_rbm_from_ellpack(E, bias.data());
+        std::vector<float> again(size_t(m) * n, 0.0f);
+        bool ordered = plan.M == m && plan.N == n && plan.Ct_max == 8 && plan.blocks.size() == (m + 7) / 8;
+        size_t pairs = 0;
+        for (const RBMBlock &b : plan.blocks) {
+            ordered &= b.colptr.size() == b.krel.size() + 1 && b.bias.size() == b.Ct && b.bias[0] == bias[b.M0];
+            for (size_t u = 0; u < b.krel.size(); ++u) {
+                ordered &= (u == 0 || b.krel[u] > b.krel[u - 1]) && b.colptr[u + 1] > b.colptr[u];
+                for (uint32_t p = b.colptr[u]; p < b.colptr[u + 1]; ++p, ++pairs) {
+                    ordered &= p == b.colptr[u] || b.pairs[p].row > b.pairs[p - 1].row;
+                    again[size_t(b.M0 + b.pairs[p].row) * n + b.krel[u]] = b.pairs[p].w;
+                }
+            }
+        }
+        size_t stored = 0;
+        for (uint32_t c : E.nnz) stored += c;
+        check(ordered && pairs == stored && std::memcmp(again.data(), W.data(), again.size() * sizeof(float)) == 0,
+              "build_rbm_from_ellpack: ordered, complete, decodes to W");
+    }
 
     if (argc == 5) {
         const uint32_t B = (uint32_t)std::atoi(argv[4]);

@@ -79,6 +79,29 @@ def main():
             out["conv%d_Ypf" % i] = ref.conv(Wc, g, X.ravel(), B, cb, False, 0).reshape(Cout, g.H_out, g.W_out, B)
         out["conv%d_W" % i], out["conv%d_X" % i], out["conv%d_b" % i] = Wc, X, cb
 
+    # row-block-merged format: the reference's build_rbm_from_ellpack on the first matrix (blocks of
+    # 8 rows and of 4), flattened as oracle.RbmArrays; and its RBM convolution (variant 3) on shapes
+    # whose batch suits this build's RBM kernel (multiples of 16, enough nonzeros per channel)
+    for ct in (8, 4):
+        R = ref.rbm_build(h, ct)
+        for key in ("block_union", "krel", "colptr", "pair_row", "pair_w"):
+            out["rbm%d_%s" % (ct, key)] = getattr(R, key)
+    rcases = [(16, 32, 12, 12, 16, (3, 3), (1, 1), (1, 1), (1, 1)),
+              (8, 24, 10, 10, 32, (3, 3), (2, 2), (1, 1), (1, 1)),
+              (32, 20, 6, 6, 16, (1, 1), (1, 1), (0, 0), (1, 1))]
+    out["rbmconv_cases"] = np.array([[c[0], c[1], c[2], c[3], c[4], *c[5], *c[6], *c[7], *c[8]] for c in rcases], dtype=np.int64)
+    for i, (Cin, Cout, H, Wi, B, k, s, p, d) in enumerate(rcases):
+        g = conv_geom(Cin, Cout, k[0], k[1], H, Wi, s, p, d)
+        Wc = rng.standard_normal((Cout, Cin * k[0] * k[1])).astype(np.float32)
+        Wc[rng.random(Wc.shape) < 0.75] = 0.0
+        X = rng.standard_normal((Cin, H, Wi, B)).astype(np.float32)
+        cb = rng.standard_normal(Cout).astype(np.float32)
+        XF = np.ascontiguousarray(X.transpose(2, 1, 0, 3))
+        for relu in (False, True):
+            Y = ref.conv(Wc, g, XF.ravel(), B, cb, relu, 3).reshape(g.W_out, g.H_out, Cout, B).transpose(2, 1, 0, 3)
+            out["rbmconv%d_Y%s" % (i, "relu" if relu else "")] = np.ascontiguousarray(Y)
+        out["rbmconv%d_W" % i], out["rbmconv%d_X" % i], out["rbmconv%d_b" % i] = Wc, X, cb
+
     path = os.path.join(HERE, "ref_vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes,", len(out), "arrays")

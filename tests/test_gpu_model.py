@@ -328,7 +328,7 @@ def test_cpp_caller_of_the_reference_headers(oracle, tmp_path):
     r = subprocess.run([exe, path, str(tmp_path / "in.bin"), str(tmp_path / "expected.bin"), str(B)],
                        capture_output=True, text=True, timeout=100)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("ok  ") == 9 and "FAIL" not in r.stdout
+    assert r.stdout.count("ok  ") == 10 and "FAIL" not in r.stdout
 
 
 def _run_device(model, ctx, X_bm):
@@ -374,3 +374,30 @@ def test_run_device_cnn(backend, ctx, tmp_path, B):
     Y = model.run(X)
     assert np.array_equal(_run_device(model, ctx, X), Y)
     assert np.array_equal(_run_device(model, ctx, X), Y)
+
+
+@pytest.mark.parametrize("B", [32, 16, 6])
+def test_model_runs_the_row_block_merged_plan(backend, oracle, tmp_path, B):
+    """The loader builds the row-block-merged plan for convolutions with Cout >= 32 and K >= 64 (the
+    reference's rule, src/sparse_onnx.cpp:499-502) and hands it to the device library.  With the RBM kernel
+    forced on every launch it fits, forbidden, and left to the library's choice, a ResNet-shaped model gives
+    the same bits, and they are the oracle chain's."""
+    from graph_oracle import run_graph
+    payload, _ = datagen.resnet18_onnx(seed=11, batch=B, hw=64, sparsity=0.8, classes=10, width=32)
+    X = np.random.default_rng(4).standard_normal((B, 3, 64, 64)).astype(np.float32)
+    outs = {}
+    try:
+        for mode in ("1", "0", None):
+            if mode is None:
+                os.environ.pop("SPARSEOPS_CONV_RBM", None)
+            else:
+                os.environ["SPARSEOPS_CONV_RBM"] = mode
+            backend.reload_tuning()
+            model = backend.SparseOnnxModel(ow.save(str(tmp_path / "r18.onnx"), payload))
+            outs[mode] = model.run(X)
+            assert np.array_equal(model.run(X), outs[mode])
+    finally:
+        os.environ.pop("SPARSEOPS_CONV_RBM", None)
+        backend.reload_tuning()
+    assert np.array_equal(outs["1"], outs["0"]) and np.array_equal(outs[None], outs["0"])
+    assert np.array_equal(outs["0"][:2], run_graph(oracle, payload, X[:2]))
