@@ -537,33 +537,96 @@ void ellpack_decode_kernel(const float *__restrict__ Wd, const uint32_t *__restr
 
 namespace {
 
-// Pass 1 of the encoder: one wave per row counts the entries with v != 0.0f.
-__global__ __launch_bounds__(256)
-void ellpack_count_kernel(const float *__restrict__ W, uint32_t m, uint32_t n, uint32_t *__restrict__ nnz)
+// The encoder's counting pass leaves one partial result per workgroup -- the longest row and the
+// number of nonzeros among the workgroup's kEncodeRowsPerBlock rows -- in a scratch buffer; a
+// one-workgroup pass folds them into the buffer's header {r, total nnz (low, high), 0}, which the
+// packing pass reads on the device, so the row pitch of the output never travels through the host.
+// Layout of the scratch buffer: header (kEncodeHeaderBytes), then one uint2 {max, sum} per workgroup.
+constexpr uint32_t kEncodeRowsPerBlock = 16;      // 4 waves x 4 rows
+constexpr uint32_t kEncodeHeaderBytes = 256;
+constexpr uint32_t kEncodeMaxCols = 1u << 28;     // 16 rows of that many columns still count in 32 bits
+
+static size_t encode_scratch_bytes(uint32_t m)
 {
-    const uint32_t lane = threadIdx.x & 63u;
-    const uint32_t nwaves = gridDim.x * 4u;
-    for (uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6); row < m; row += nwaves) {
+    return kEncodeHeaderBytes + (size_t)so_ceil_div(m, kEncodeRowsPerBlock) * sizeof(uint2);
+}
+
+// Pass 1: one wave per row counts the entries with v != 0.0f; the workgroup's maximum and sum go
+// to partial[blockIdx.x].
+__global__ __launch_bounds__(256)
+void ellpack_count_kernel(const float *__restrict__ W, uint32_t m, uint32_t n, uint32_t *__restrict__ nnz,
+                          uint2 *__restrict__ partial)
+{
+    __shared__ uint32_t wmax[4], wsum[4];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint32_t vmax = 0, vsum = 0;
+    for (uint32_t k = 0; k < kEncodeRowsPerBlock / 4u; ++k) {
+        const uint32_t row = blockIdx.x * kEncodeRowsPerBlock + k * 4u + wave;
+        if (row >= m) break;
         const float *wr = W + (size_t)row * n;
         uint32_t c = 0;
         for (uint32_t j = lane; j < n; j += 64u) c += wr[j] != 0.0f ? 1u : 0u;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
         if (lane == 0) nnz[row] = c;
+        vmax = max(vmax, c);
+        vsum += c;
+    }
+    if (lane == 0) { wmax[wave] = vmax; wsum[wave] = vsum; }
+    __syncthreads();
+    if (threadIdx.x == 0)
+        partial[blockIdx.x] = make_uint2(max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])),
+                                         wsum[0] + wsum[1] + wsum[2] + wsum[3]);
+}
+
+// Folds the partials into header = {r, total nnz low word, high word, 0}.  One workgroup.
+__global__ __launch_bounds__(1024)
+void ellpack_count_fold_kernel(const uint2 *__restrict__ partial, uint32_t nblocks, uint32_t *__restrict__ header)
+{
+    __shared__ uint32_t smax[16];
+    __shared__ unsigned long long ssum[16];
+    uint32_t vmax = 0;
+    unsigned long long vsum = 0;
+    for (uint32_t i = threadIdx.x; i < nblocks; i += 1024u) {
+        const uint2 p = partial[i];
+        vmax = max(vmax, p.x);
+        vsum += p.y;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        vmax = max(vmax, (uint32_t)__shfl_xor(vmax, off, 64));
+        vsum += __shfl_xor(vsum, off, 64);
+    }
+    if ((threadIdx.x & 63u) == 0) { smax[threadIdx.x >> 6] = vmax; ssum[threadIdx.x >> 6] = vsum; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; ++w) { vmax = max(vmax, smax[w]); vsum += ssum[w]; }
+        header[0] = vmax;
+        header[1] = (uint32_t)vsum;
+        header[2] = (uint32_t)(vsum >> 32);
+        header[3] = 0u;
     }
 }
 
-// Pass 2: one wave per row packs (value, column) in ascending column order.  For each group of
-// 64 columns the lanes that hold a nonzero get consecutive slots (a prefix count over the wave's
-// ballot), so the order inside the row is the column order.  Wd/idx were zero-filled before.
+// Pass 2: one wave per row packs (value, column) in ascending column order with row pitch
+// r = header[0], then zero-fills the row's remaining slots.  For each group of 64 columns the lanes
+// that hold a nonzero get consecutive slots (a prefix count over the wave's ballot), so the order
+// inside the row is the column order.  Writes nothing when r exceeds r_cap (the caller's arrays
+// hold m * r_cap slots); the wave that owns the last row also clears `tail_words` words after the
+// arrays' last slot.
 __global__ __launch_bounds__(256)
-void ellpack_pack_kernel(const float *__restrict__ W, uint32_t m, uint32_t n, uint32_t r,
-                         float *__restrict__ Wd, uint32_t *__restrict__ idx)
+void ellpack_pack_kernel(const float *__restrict__ W, uint32_t m, uint32_t n, const uint32_t *__restrict__ header,
+                         uint32_t r_cap, const uint32_t *__restrict__ nnz, float *__restrict__ Wd,
+                         uint32_t *__restrict__ idx, uint32_t tail_words)
 {
+    const uint32_t r = header[0];
+    if (r > r_cap) return;
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t nwaves = gridDim.x * 4u;
     for (uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6); row < m; row += nwaves) {
         const float *wr = W + (size_t)row * n;
+        float *wd = Wd + (size_t)row * r;
+        uint32_t *ix = idx + (size_t)row * r;
         uint32_t base = 0;
         for (uint32_t j0 = 0; j0 < n; j0 += 64u) {
             const uint32_t j = j0 + lane;
@@ -572,12 +635,38 @@ void ellpack_pack_kernel(const float *__restrict__ W, uint32_t m, uint32_t n, ui
             const uint64_t mask = __ballot(keep);
             if (keep) {
                 const uint32_t pos = base + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-                Wd[(size_t)row * r + pos] = v;
-                idx[(size_t)row * r + pos] = j;
+                wd[pos] = v;
+                ix[pos] = j;
             }
             base += (uint32_t)__popcll(mask);
         }
+        const uint32_t end = row + 1 == m ? r + tail_words : r;
+        for (uint32_t k = nnz[row] + lane; k < end; k += 64u) { wd[k] = 0.0f; ix[k] = 0u; }
     }
+}
+
+// The three passes on the context's stream.  `scratch` holds encode_scratch_bytes(m) bytes; dWd and
+// dIdx hold m * r_cap slots (+ tail_words).
+so_status encode_launch(so_ctx *ctx, const float *dDense, uint32_t m, uint32_t n, void *scratch, uint32_t r_cap,
+                        uint32_t *dNnz, float *dWd, uint32_t *dIdx, uint32_t tail_words, bool count, bool pack)
+{
+    uint32_t *header = (uint32_t *)scratch;
+    uint2 *partial = (uint2 *)((char *)scratch + kEncodeHeaderBytes);
+    const uint32_t nblocks = so_ceil_div(m, kEncodeRowsPerBlock);
+    if (count) {
+        if (nblocks) {
+            ellpack_count_kernel<<<nblocks, 256, 0, ctx->stream>>>(dDense, m, n, dNnz, partial);
+            SO_LAUNCH_CHECK();
+        }
+        ellpack_count_fold_kernel<<<1, 1024, 0, ctx->stream>>>(partial, nblocks, header);
+        SO_LAUNCH_CHECK();
+    }
+    if (pack && m) {
+        const uint32_t blocks = std::max(1u, std::min(so_ceil_div(m, 4u), 16u * (uint32_t)ctx->compute_units));
+        ellpack_pack_kernel<<<blocks, 256, 0, ctx->stream>>>(dDense, m, n, header, r_cap, dNnz, dWd, dIdx, tail_words);
+        SO_LAUNCH_CHECK();
+    }
+    return SO_OK;
 }
 
 } // namespace
@@ -587,32 +676,35 @@ extern "C" so_status so_ellpack_encode(so_ctx *ctx, const float *dDense, uint32_
     SO_REQUIRE(ctx && out, "so_ellpack_encode: null argument");
     *out = nullptr;
     SO_REQUIRE(dDense != nullptr || (uint64_t)m * n == 0, "so_ellpack_encode: null matrix");
+    SO_REQUIRE(n <= kEncodeMaxCols, "so_ellpack_encode: at most %u columns", kEncodeMaxCols);
     so_ellpack *E = new (std::nothrow) so_ellpack();
     if (!E) { so_set_error("so_ellpack_encode: host allocation failed"); return SO_ERR_OOM; }
     E->m = m; E->n = n;
     E->layouts = SO_LAYOUT_ROW;
-    std::vector<uint32_t> nnz(m, 0);
-    void *p = nullptr;
+    void *p = nullptr, *scratch = nullptr;
+    uint32_t header[4] = {0, 0, 0, 0};
     so_status s = so_malloc(ctx, (size_t)m * sizeof(uint32_t) + 16, &p);
-    if (s == SO_OK) { E->d_nnz = (uint32_t *)p; s = so_fill_zero(ctx, p, (size_t)m * sizeof(uint32_t) + 16); }
-    const uint32_t blocks = std::max(1u, std::min(so_ceil_div(m, 4u), 16u * (uint32_t)ctx->compute_units));
-    if (s == SO_OK && m && n) {
-        ellpack_count_kernel<<<blocks, 256, 0, ctx->stream>>>(dDense, m, n, E->d_nnz);
-        if (hipGetLastError() != hipSuccess) { so_set_error("so_ellpack_encode: launch failed"); s = SO_ERR_HIP; }
-    }
-    if (s == SO_OK && m) s = so_d2h(ctx, nnz.data(), E->d_nnz, (size_t)m * sizeof(uint32_t));
+    if (s == SO_OK) { E->d_nnz = (uint32_t *)p; s = so_fill_zero(ctx, (char *)p + (size_t)m * sizeof(uint32_t), 16); }
+    if (s == SO_OK) s = so_malloc(ctx, encode_scratch_bytes(m), &scratch);
+    if (s == SO_OK) s = encode_launch(ctx, dDense, m, n, scratch, 0, E->d_nnz, nullptr, nullptr, 0, true, false);
+    if (s == SO_OK) s = so_d2h(ctx, header, scratch, sizeof header);
     if (s == SO_OK) {
-        for (uint32_t c : nnz) { E->total_nnz += c; E->max_nnz = std::max(E->max_nnz, c); }
-        E->r = E->max_nnz;                               // r = longest row (src/ellpack_encoder.cpp:10-17)
+        E->r = E->max_nnz = header[0];                   // r = longest row (src/ellpack_encoder.cpp:10-17)
+        E->total_nnz = (uint64_t)header[1] | ((uint64_t)header[2] << 32);
         const size_t bytes = (size_t)m * E->r * sizeof(float) + 16;
         s = so_malloc(ctx, bytes, &p);
-        if (s == SO_OK) { E->d_Wd = (float *)p; s = so_fill_zero(ctx, p, bytes); }
-        if (s == SO_OK) s = so_malloc(ctx, bytes, &p);
-        if (s == SO_OK) { E->d_idx = (uint32_t *)p; s = so_fill_zero(ctx, p, bytes); }
+        if (s == SO_OK) { E->d_Wd = (float *)p; s = so_malloc(ctx, bytes, &p); }
+        if (s == SO_OK) E->d_idx = (uint32_t *)p;
+        if (s == SO_OK && (size_t)m * E->r == 0) {
+            s = so_fill_zero(ctx, E->d_Wd, 16);
+            if (s == SO_OK) s = so_fill_zero(ctx, E->d_idx, 16);
+        }
     }
-    if (s == SO_OK && E->r) {
-        ellpack_pack_kernel<<<blocks, 256, 0, ctx->stream>>>(dDense, m, n, E->r, E->d_Wd, E->d_idx);
-        if (hipGetLastError() != hipSuccess) { so_set_error("so_ellpack_encode: launch failed"); s = SO_ERR_HIP; }
+    if (s == SO_OK && (size_t)m * E->r != 0)
+        s = encode_launch(ctx, dDense, m, n, scratch, E->r, E->d_nnz, E->d_Wd, E->d_idx, 4, false, true);
+    if (scratch) {
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipFree(scratch);
     }
     if (s != SO_OK) {
         (void)so_ellpack_free(ctx, E);
