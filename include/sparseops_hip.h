@@ -144,6 +144,21 @@ so_status so_ellpack_download(so_ctx *ctx, const so_ellpack *E, int layout,
  * column order, so -0.0f is dropped and NaN kept; r = longest row; zero padding).
  * Other layouts: download and upload again with the layouts wanted. */
 so_status so_ellpack_encode(so_ctx *ctx, const float *dDense, uint32_t m, uint32_t n, so_ellpack **out);
+/* so_ellpack_encode for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Calls no hipMalloc,
+ * hipFree or allocating routine: the caller brings the outputs -- dNnz[m], dWd and dIdx of
+ * m * r_cap slots each -- and the counting pass's partial results live in a static device array of
+ * the library (524 544 bytes per GPU, held until the process ends), which limits a call to
+ * 1 048 576 rows (more: SO_ERR_INVALID).  Output: dNnz[i] = nonzeros of row i, and dWd/dIdx packed
+ * with row pitch r = the longest row, i.e. the first m * r slots hold exactly the arrays
+ * so_ellpack_encode produces.  When r exceeds r_cap nothing is packed (dNnz is still valid).
+ * r_out / total_nnz_out (host, may be NULL) receive r and the nonzero count; asking for either makes
+ * the call wait for the device, and the call then fails with SO_ERR_INVALID when r > r_cap; with
+ * both NULL it returns without waiting.  All calls on one GPU share the array: calls that overlap
+ * on one GPU (two contexts, two threads) race. */
+so_status so_ellpack_encode_noalloc(so_ctx *ctx, const float *dDense, uint32_t m, uint32_t n,
+                                    uint32_t r_cap, float *dWd, uint32_t *dIdx, uint32_t *dNnz,
+                                    uint32_t *r_out, uint64_t *total_nnz_out);
 /* decode_from_ellpack (src/ellpack_encoder.cpp:46-60) on the device: dDense [m x n] row-major
  * is zeroed, then the first nnz[i] entries of every row are scattered into it. */
 so_status so_ellpack_decode(so_ctx *ctx, const so_ellpack *E, float *dDense);

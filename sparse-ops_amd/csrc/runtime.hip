@@ -8,6 +8,13 @@
 
 static thread_local std::string g_last_error;
 
+// Scratch memory of so_ellpack_encode_noalloc: the counting pass's header and per-workgroup partial
+// results (layout further down, at the encoder).  Every GPU the library runs on holds its own copy
+// at its own address; host code never uses this name as a pointer, only the address that so_init
+// looks up for the context's device.
+constexpr size_t kStaticScratchBytes = 256 + 65536 * 8;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 void so_set_error(const char *fmt, ...)
 {
     char buf[512];
@@ -97,6 +104,13 @@ extern "C" so_status so_init(int device, so_ctx **out)
     if (e == hipSuccess) e = hipEventCreate(&ctx->ev1);
     if (e != hipSuccess) {
         so_set_error("so_init: stream/event creation failed: %s", hipGetErrorString(e));
+        so_destroy(ctx);
+        return SO_ERR_HIP;
+    }
+    // this device's copy of the static scratch array (the device is current)
+    e = hipGetSymbolAddress(&ctx->static_scratch, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ctx->static_scratch == nullptr) {
+        so_set_error("so_init: hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
         so_destroy(ctx);
         return SO_ERR_HIP;
     }
@@ -543,8 +557,11 @@ namespace {
 // packing pass reads on the device, so the row pitch of the output never travels through the host.
 // Layout of the scratch buffer: header (kEncodeHeaderBytes), then one uint2 {max, sum} per workgroup.
 constexpr uint32_t kEncodeRowsPerBlock = 16;      // 4 waves x 4 rows
+constexpr uint32_t kEncodeMaxBlocks = 65536;      // workgroups whose partials the static scratch array holds
 constexpr uint32_t kEncodeHeaderBytes = 256;
 constexpr uint32_t kEncodeMaxCols = 1u << 28;     // 16 rows of that many columns still count in 32 bits
+constexpr size_t kEncodeScratchBytes = kEncodeHeaderBytes + (size_t)kEncodeMaxBlocks * sizeof(uint2);
+static_assert(kEncodeScratchBytes <= kStaticScratchBytes, "the static scratch array holds the encoder's partials");
 
 static size_t encode_scratch_bytes(uint32_t m)
 {
@@ -711,6 +728,33 @@ extern "C" so_status so_ellpack_encode(so_ctx *ctx, const float *dDense, uint32_
         return s;
     }
     *out = E;
+    return SO_OK;
+}
+
+extern "C" so_status so_ellpack_encode_noalloc(so_ctx *ctx, const float *dDense, uint32_t m, uint32_t n, uint32_t r_cap,
+                                              float *dWd, uint32_t *dIdx, uint32_t *dNnz, uint32_t *r_out,
+                                              uint64_t *total_nnz_out)
+{
+    SO_REQUIRE(ctx != nullptr, "so_ellpack_encode_noalloc: ctx is null");
+    SO_REQUIRE(dDense != nullptr || (uint64_t)m * n == 0, "so_ellpack_encode_noalloc: null matrix");
+    SO_REQUIRE(n <= kEncodeMaxCols, "so_ellpack_encode_noalloc: at most %u columns", kEncodeMaxCols);
+    SO_REQUIRE(so_ceil_div(m, kEncodeRowsPerBlock) <= kEncodeMaxBlocks,
+               "so_ellpack_encode_noalloc: %u rows need %u partial results, the static scratch array holds %u (at most %u rows)",
+               m, so_ceil_div(m, kEncodeRowsPerBlock), kEncodeMaxBlocks, kEncodeMaxBlocks * kEncodeRowsPerBlock);
+    SO_REQUIRE(m == 0 || dNnz != nullptr, "so_ellpack_encode_noalloc: dNnz is null");
+    SO_REQUIRE((uint64_t)m * r_cap == 0 || (dWd != nullptr && dIdx != nullptr), "so_ellpack_encode_noalloc: dWd/dIdx is null");
+    SO_REQUIRE(ctx->static_scratch != nullptr, "so_ellpack_encode_noalloc: the context has no scratch address");
+    const so_status s = encode_launch(ctx, dDense, m, n, ctx->static_scratch, r_cap, dNnz, dWd, dIdx, 0, true,
+                                      (uint64_t)m * r_cap != 0);
+    if (s != SO_OK || (!r_out && !total_nnz_out)) return s;
+    SO_REQUIRE(!ctx->capturing, "so_ellpack_encode_noalloc: r_out/total_nnz_out need a wait, which a graph recording forbids");
+    uint32_t header[4] = {0, 0, 0, 0};
+    SO_HIP(hipMemcpyAsync(header, ctx->static_scratch, sizeof header, hipMemcpyDeviceToHost, ctx->stream));
+    SO_HIP(hipStreamSynchronize(ctx->stream));
+    if (r_out) *r_out = header[0];
+    if (total_nnz_out) *total_nnz_out = (uint64_t)header[1] | ((uint64_t)header[2] << 32);
+    SO_REQUIRE(header[0] <= r_cap, "so_ellpack_encode_noalloc: the longest row has %u nonzeros, dWd/dIdx hold %u per row (nothing was packed)",
+               header[0], r_cap);
     return SO_OK;
 }
 

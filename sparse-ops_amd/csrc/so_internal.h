@@ -30,6 +30,7 @@ struct so_ctx {
     int compute_units = 0;
     int max_lds_bytes = 0;   // largest LDS allocation one workgroup may ask for
     bool capturing = false;
+    void *static_scratch = nullptr;   // this device's address of the library's static scratch array (so_ellpack_encode_noalloc)
     std::string name;
     so_tuning tune;
     std::vector<const void *> big_lds_kernels;   // kernels already allowed max_lds_bytes of dynamic LDS on this device

@@ -20,7 +20,7 @@ LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS, LAYOUT_TILED = 1, 2, 4, 8
 SYMBOLS = (
     "so_device_count so_init so_destroy so_last_error so_device_info so_tuning_reload so_malloc so_free so_h2d so_d2h "
     "so_d2d so_fill_zero so_sync so_timer_begin so_timer_end so_ellpack_upload so_ellpack_free "
-    "so_ellpack_dims so_ellpack_download so_ellpack_decode so_ellpack_encode so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
+    "so_ellpack_dims so_ellpack_download so_ellpack_decode so_ellpack_encode so_ellpack_encode_noalloc so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
     "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_copy_rows so_graph_begin so_graph_end "
     "so_graph_launch so_graph_free so_rbm_upload so_rbm_free so_rbm_dims so_conv_plan_set_rbm so_conv_plan_rbm_info").split()
 
@@ -79,6 +79,7 @@ def load_library(path=None):
         "so_ellpack_download": [_vp, _vp, ct.c_int, _vp, _vp, _vp],
         "so_ellpack_decode": [_vp, _vp, _vp],
         "so_ellpack_encode": [_vp, _vp, _u32, _u32, ct.POINTER(_vp)],
+        "so_ellpack_encode_noalloc": [_vp, _vp, _u32, _u32, _u32, _vp, _vp, _vp, ct.POINTER(_u32), ct.POINTER(ct.c_uint64)],
         "so_matmul": [_vp, _vp, _vp, _u32, _vp, _vp, ct.c_int],
         "so_matvec": [_vp, _vp, _vp, _vp, _vp, ct.c_int],
         "so_conv_plan_create": [_vp, _vp, ct.POINTER(ConvGeom), ct.POINTER(_vp)],
@@ -252,6 +253,15 @@ class Context:
         r = ct.c_uint32()
         self._ck(self.lib.so_ellpack_dims(h, None, None, ct.byref(r), None, None))
         return DeviceEllpack(self, h.value, m, n, r.value)
+
+    def encode_dense_noalloc(self, dW, m, n, r_cap, dWd, dIdx, dNnz, want_counts=True):
+        """so_ellpack_encode_noalloc into the caller's DeviceArrays -> (r, total nnz), or None without a wait."""
+        r, total = ct.c_uint32(), ct.c_uint64()
+        self._ck(self.lib.so_ellpack_encode_noalloc(
+            self.h, dW.ptr if dW is not None else None, m, n, r_cap, dWd.ptr if dWd is not None else None,
+            dIdx.ptr if dIdx is not None else None, dNnz.ptr if dNnz is not None else None,
+            ct.byref(r) if want_counts else None, ct.byref(total) if want_counts else None))
+        return (r.value, total.value) if want_counts else None
 
     def matmul(self, E, dX, C, dBias, dY, act="none"):
         self._ck(self.lib.so_matmul(self.h, E.h, dX.ptr, C, dBias.ptr if dBias else None, dY.ptr, ACT[act]))
