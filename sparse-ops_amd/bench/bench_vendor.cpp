@@ -3,12 +3,17 @@
 // same flags (--M --N --C --sparsity --runs --seed --irregular), same data recipe
 // (N(0,1) values under an i.i.d. Bernoulli mask, optionally a dense last row; X ~ U(-1,1);
 // no bias; benchmark-mkl/common/data_gen.cpp:23-96), 1 warm-up then the median of --runs,
-// reported in microseconds.  The comparators are the ROCm counterparts of the reference's:
+// reported in microseconds.  Random numbers come from std::mt19937_64 through explicit
+// transforms (53-bit uniforms, Box-Muller normals): the standard library's distribution
+// classes may differ between implementations, these do not.  --ellpack-file <path> replaces
+// the generated matrix by one written by python/datagen.py's save_ellpack (any of the
+// benchmark configurations), so the very same matrix runs here and in bench.py.  The comparators are the ROCm counterparts of the reference's:
 // rocSPARSE CSR SpMM / SpMV for MKL sparse, rocBLAS SGEMM / SGEMV for the dense BLAS, and
 // this library's so_matmul (row-per-wave and LDS-staged) / so_matvec for "Ellpack".
 //
 //   bench_vendor matmul --M 4096 --N 4096 --C 256 --sparsity 0.9 --runs 100
 //   bench_vendor matvec --M 16384 --N 16384 --sparsity 0.95 --runs 100
+//   bench_vendor matmul --ellpack-file config3.ellpack --C 256 --runs 100
 #include <hip/hip_runtime.h>
 #include <rocblas/rocblas.h>
 #include <rocsparse/rocsparse.h>
@@ -42,18 +47,71 @@ struct Host {
     std::vector<uint32_t> idx, nnz;
 };
 
+// Explicit transforms of the generator's 64-bit outputs.
+inline double uniform01(std::mt19937_64 &rng) { return double(rng() >> 11) * (1.0 / 9007199254740992.0); }   // [0, 1), 53 bits
+inline float normal01(std::mt19937_64 &rng)
+{
+    const double u1 = 1.0 - uniform01(rng), u2 = uniform01(rng);                                              // u1 in (0, 1]
+    return float(std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586476925 * u2));
+}
+
+// CSR and ELLPACK views of the dense matrix in h.W.
+void derive_formats(Host &h);
+
 Host generate(int64_t M, int64_t N, double sparsity, uint64_t seed, bool irregular)
 {
     Host h;
     h.M = M; h.N = N;
     h.W.assign(size_t(M) * N, 0.0f);
     std::mt19937_64 rng(seed);
-    std::normal_distribution<float> val(0.0f, 1.0f);
-    std::uniform_real_distribution<double> coin(0.0, 1.0);
     const double keep = 1.0 - sparsity;
     for (int64_t i = 0; i < M; ++i)
         for (int64_t j = 0; j < N; ++j)
-            if ((irregular && i == M - 1) || coin(rng) < keep) h.W[size_t(i) * N + j] = val(rng);
+            if ((irregular && i == M - 1) || uniform01(rng) < keep) h.W[size_t(i) * N + j] = normal01(rng);
+    derive_formats(h);
+    return h;
+}
+
+// A matrix written by python/datagen.py save_ellpack: "SOELLPK1", uint32 m, n, r, 0, then nnz[m],
+// idx[m*r] (uint32) and Wd[m*r] (float), little endian.
+Host load_ellpack_file(const char *path)
+{
+    std::FILE *f = std::fopen(path, "rb");
+    if (!f) { std::fprintf(stderr, "cannot open %s\n", path); std::exit(2); }
+    char magic[8];
+    uint32_t hdr[4];
+    if (std::fread(magic, 1, 8, f) != 8 || std::memcmp(magic, "SOELLPK1", 8) != 0 || std::fread(hdr, 4, 4, f) != 4) {
+        std::fprintf(stderr, "%s: not an ELLPACK file\n", path);
+        std::exit(2);
+    }
+    Host h;
+    h.M = hdr[0]; h.N = hdr[1];
+    const uint32_t r = hdr[2];
+    const size_t slots = size_t(h.M) * r;
+    std::vector<uint32_t> nnz(h.M), idx(slots);
+    std::vector<float> Wd(slots);
+    if (std::fread(nnz.data(), 4, nnz.size(), f) != nnz.size() || std::fread(idx.data(), 4, slots, f) != slots ||
+        std::fread(Wd.data(), 4, slots, f) != slots) {
+        std::fprintf(stderr, "%s: truncated\n", path);
+        std::exit(2);
+    }
+    std::fclose(f);
+    h.W.assign(size_t(h.M) * h.N, 0.0f);
+    for (int64_t i = 0; i < h.M; ++i) {
+        if (nnz[i] > r) { std::fprintf(stderr, "%s: nnz[%lld] exceeds r\n", path, (long long)i); std::exit(2); }
+        for (uint32_t k = 0; k < nnz[i]; ++k) {
+            const uint32_t j = idx[size_t(i) * r + k];
+            if (j >= h.N) { std::fprintf(stderr, "%s: column out of range\n", path); std::exit(2); }
+            h.W[size_t(i) * h.N + j] = Wd[size_t(i) * r + k];
+        }
+    }
+    derive_formats(h);
+    return h;
+}
+
+void derive_formats(Host &h)
+{
+    const int64_t M = h.M, N = h.N;
     h.row_ptr.assign(M + 1, 0);
     h.nnz.assign(M, 0);
     for (int64_t i = 0; i < M; ++i) {
@@ -71,7 +129,6 @@ Host generate(int64_t M, int64_t N, double sparsity, uint64_t seed, bool irregul
             h.Wd[size_t(i) * h.r + k] = h.values[h.row_ptr[i] + k];
             h.idx[size_t(i) * h.r + k] = uint32_t(h.col_ind[h.row_ptr[i] + k]);
         }
-    return h;
 }
 
 template <typename T>
@@ -134,7 +191,7 @@ int main(int argc, char **argv)
 {
     if (argc < 2 || (std::strcmp(argv[1], "matmul") && std::strcmp(argv[1], "matvec"))) {
         std::fprintf(stderr, "usage: %s matmul|matvec --M <rows> --N <cols> [--C <cols of X>] --sparsity <p> --runs <r> "
-                             "--seed <s> --irregular <0|1> [--device <id>]\n", argv[0]);
+                             "--seed <s> --irregular <0|1> [--device <id>] [--ellpack-file <path>]\n", argv[0]);
         return 1;
     }
     const bool matmul = !std::strcmp(argv[1], "matmul");
@@ -144,6 +201,7 @@ int main(int argc, char **argv)
     uint64_t seed = 42;
     bool irregular = false;
     int device = 0;
+    const char *ellpack_file = nullptr;
     for (int i = 2; i < argc; ++i) {
         const std::string a = argv[i];
         if (i + 1 >= argc) { std::fprintf(stderr, "incomplete arg: %s\n", a.c_str()); return 1; }
@@ -155,19 +213,24 @@ int main(int argc, char **argv)
         else if (a == "--seed") seed = std::stoull(argv[++i]);
         else if (a == "--irregular") irregular = std::stoi(argv[++i]) != 0;
         else if (a == "--device") device = std::stoi(argv[++i]);
+        else if (a == "--ellpack-file") ellpack_file = argv[++i];
         else { std::fprintf(stderr, "unknown arg: %s\n", a.c_str()); return 1; }
     }
     if (!matmul) C = 1;
+    Host h = ellpack_file ? load_ellpack_file(ellpack_file) : generate(M, N, sparsity, seed, irregular);
+    if (ellpack_file) {
+        M = h.M; N = h.N;
+        sparsity = 1.0 - double(h.values.size()) / std::max<double>(1.0, double(M) * double(N));
+        std::printf("Matrix file:     %s\n", ellpack_file);
+    }
     std::printf("=== Sparse %s benchmark (MI355X) ===\nMatrix dims:     %lld x %lld\nDense cols C:    %d\nSparsity:        %g\n"
                 "Repetitions:     %d\nRNG seed:        %llu\nIrregular last row: %d\n\n",
                 matmul ? "MatMul" : "MatVec", (long long)M, (long long)N, C, sparsity, runs, (unsigned long long)seed, int(irregular));
 
-    Host h = generate(M, N, sparsity, seed, irregular);
     std::vector<float> X(size_t(N) * C);
     {
         std::mt19937_64 rng(seed);
-        std::uniform_real_distribution<float> dist(-1.0f, 1.0f);
-        for (auto &v : X) v = dist(rng);
+        for (auto &v : X) v = float(2.0 * uniform01(rng) - 1.0);
     }
     const size_t nnz_total = h.values.size();
     std::printf("nnz %zu, ELLPACK r %u (padding %.2fx)\n\n", nnz_total, h.r, nnz_total ? double(M) * h.r / nnz_total : 0.0);

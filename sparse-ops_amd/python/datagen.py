@@ -21,6 +21,28 @@ class EllpackHost:
         return int(self.nnz.sum(dtype=np.int64))
 
 
+def save_ellpack(path, E):
+    """Write E in the format bench/bench_vendor --ellpack-file reads: b"SOELLPK1", uint32 m, n, r, 0,
+    then nnz[m], idx[m*r] (uint32) and Wd[m*r] (float32), little endian."""
+    with open(path, "wb") as f:
+        f.write(b"SOELLPK1")
+        f.write(np.array([E.m, E.n, E.r, 0], dtype="<u4").tobytes())
+        f.write(E.nnz.astype("<u4").tobytes())
+        f.write(E.idx.astype("<u4").tobytes())
+        f.write(E.Wd.astype("<f4").tobytes())
+
+
+def load_ellpack(path):
+    with open(path, "rb") as f:
+        if f.read(8) != b"SOELLPK1":
+            raise ValueError("%s is not an ELLPACK file" % path)
+        m, n, r, _ = np.frombuffer(f.read(16), dtype="<u4")
+        nnz = np.frombuffer(f.read(4 * int(m)), dtype="<u4")
+        idx = np.frombuffer(f.read(4 * int(m) * int(r)), dtype="<u4")
+        Wd = np.frombuffer(f.read(4 * int(m) * int(r)), dtype="<f4")
+    return EllpackHost(m, n, r, Wd, idx, nnz)
+
+
 def encode_dense(W):
     """numpy ELLPACK encoder: same layout rules as convert_to_ellpack
     (src/ellpack_encoder.cpp:6-44), vectorised."""
