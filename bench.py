@@ -25,21 +25,29 @@ import tempfile
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for _p in (os.path.join(ROOT, "sparse-ops_amd"), os.path.join(ROOT, "sparse-ops_amd", "python")):
+for _p in (os.path.join(ROOT, "sparse-ops_amd"), os.path.join(ROOT, "sparse-ops_amd", "python"),
+           os.path.join(ROOT, "sparse-ops_amd", "bench")):
     sys.path.insert(0, _p)
 
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
-VALU_FP32_PEAK_TF = 157.3    # MI355X vector fp32 (packed FMA); 78.6 with plain v_fma_f32
-LDS_OPERAND_PEAK_TF = 39.3   # 256 CUs x 128 B/clk of LDS reads x 2.4 GHz / 4 B per multiply-add x 2 flop
-# HBM-side bytes per launch of the headline kernel, from two rocprofv3 --pmc runs
-# (FETCH_SIZE, WRITE_SIZE) scaled by a plain copy of known size; see the pmc summary
-# under profiles/.  None until measured for the kernel that currently runs.
-MEASURED_TRAFFIC_BYTES = 57_500_000   # ellpack_matmul_tiled_kernel: 53.3 MB fetched + 4.19 MB written
-# the same counters for the two matvec kernels (profiles/bench_all_kernels__pmc_hbm_bytes.txt)
-MEASURED_MATVEC_TRAFFIC = {"ellpack_matvec 16384x16384, 95% Bernoulli": 112_300_000,
-                           "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048": 69_800_000}
+VALU_FP32_PEAK_TF = 157.3    # MI355X vector fp32; plain v_fma_f32 reaches 107 of its 128 multiply-adds per clock and CU,
+                             # the DPP form the quad layout needs 58 (profiles/lds_valu_rates__probe.txt)
+LDS_OPERAND_PEAK_TF = 78.6   # 256 CUs x 256 B/clk of ds_read_b128 (measured 255) x 2.4 GHz / 4 B per multiply-add x 2 flop
+# HBM-side bytes per launch, per kernel: measured with two rocprofv3 --pmc runs (FETCH_SIZE,
+# WRITE_SIZE) scaled by a plain copy of known size and kept, keyed by kernel name and together with a
+# hash of the kernel's sources, in this table (written by sparse-ops_amd/bench/pmc_summary.py traffic).
+# A kernel that is not in the table, or whose sources have changed since, reports null.
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+HEADLINE_KERNEL = "ellpack_matmul_tiled_kernel<0>"
+MATVEC_KERNELS = {"ellpack_matvec 16384x16384, 95% Bernoulli": ("matvec_rows_kernel", "matvec 16384^2 uniform"),
+                  "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048": ("matvec_binned_kernel", "matvec 16384^2 zipf")}
+
+
+def measured_traffic(kernel, workload=None):
+    from pmc_summary import lookup_traffic
+    return lookup_traffic(TRAFFIC_TABLE, kernel, workload)
 
 
 def log(*a):
@@ -80,6 +88,29 @@ def time_launches(ctx, fn, steps, warmup):
     ctx.sync()
     wall = time.perf_counter() - t0
     return wall, ev_ms / steps
+
+
+def time_groups(ctx, fn, groups, per_group):
+    """-> per-launch microseconds of `groups` event-bracketed groups of `per_group` back-to-back launches
+    (the clocks are settled by the caller's earlier time_launches)."""
+    for _ in range(per_group):
+        fn()
+    ctx.sync()
+    out = []
+    for _ in range(groups):
+        ctx.timer_begin()
+        for _ in range(per_group):
+            fn()
+        out.append(ctx.timer_end() * 1e3 / per_group)
+    return out
+
+
+def host_has_avx512f():
+    try:
+        with open("/proc/cpuinfo") as f:
+            return "avx512f" in f.read()
+    except OSError:
+        return False
 
 
 def cpu_baseline_matmul(E, X, bias, y_gpu, budget_s=15.0):
@@ -144,7 +175,9 @@ def cpu_baseline_matmul(E, X, bias, y_gpu, budget_s=15.0):
     return {
         "value": round(flops / med / 1e9, 2), "unit": "nnz-GFLOP/s", "cores": threads, "kind": kind,
         "sample": "same 4096x4096 r=410 C=256 matmul, 1 warm-up + median of %d runs (%.2f ms each)" % (len(times), med * 1e3),
-        "ms_per_step": round(med * 1e3, 4), "cpu_model": model, "nnz_gflops_by_threads": by_threads,
+        "ms_per_step": round(med * 1e3, 4), "ms_per_step_min": round(min(times) * 1e3, 4), "cpu_model": model,
+        "avx512f": host_has_avx512f(),       # without it the reference takes its scalar path (src/ellpack_matmul.cpp:80-90)
+        "nnz_gflops_by_threads": by_threads,
         "gpu_bit_exact_vs_cpu": bool(np.array_equal(Ycpu, y_gpu)),
         "gpu_max_rel_err_vs_cpu": float(np.abs(Ycpu.astype(np.float64) - y_gpu).max() / np.abs(Ycpu).max()),
     }
@@ -189,7 +222,8 @@ def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup
     nbytes = 8 * E.total_nnz + 4 * E.m + 4 * E.m + 4 * E.n + 4 * E.m
     out = {"workload": name, "m": E.m, "n": E.n, "r": E.r, "nnz": E.total_nnz, "us_per_launch": round(ms * 1e3, 2),
            "alg_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1), "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
-           "padded_bytes": 8 * E.m * E.r, "traffic": MEASURED_MATVEC_TRAFFIC.get(name)}
+           "padded_bytes": 8 * E.m * E.r,
+           "traffic": measured_traffic(*MATVEC_KERNELS[name]) if name in MATVEC_KERNELS else None}
     if with_cpu:
         out["cpu_baseline"] = cpu_baseline_matvec(E, x, b, dy.download(), nbytes)
     # Cache-cold figure: the streamed arrays (66-108 MB) fit the 256 MB Infinity Cache when the
@@ -278,24 +312,38 @@ def bench_mlp(steps, warmup, with_cpu=True):
             "nnz_gflops_device_resident": round(model.nnz_flops_per_sample() * 256 / (dev_ms * 1e-3) / 1e9, 1)}
 
 
-def cpu_baseline_cnn(payload, model, sample=4):
-    """The same graph, layer by layer, with the plain-C restatement of the reference's conv /
-    pool / add / FC kernels on the host cores (the reference's own model runtime needs
-    libprotobuf and is not buildable here, hence kind "port"), on a bounded sample of the batch.
-    Also compares the GPU's output for those images with the CPU's, bit for bit."""
+def cpu_baseline_cnn(payload, model):
+    """The same graph on the host cores over the whole batch of 32: every convolution with the
+    reference's own conv2d_rbm_fmajor_implicit (its variant that is right for strided layers) and the
+    classifier with its ellpack_matmul, both from oracle/_ref; max-pool, residual adds and the global
+    average pool with the plain-C port (the reference's versions are private members of a class whose
+    constructor needs libprotobuf).  1 warm-up pass, median of 3, kernel time only (the layout shuffles
+    between the two libraries' conventions are not counted) -- the reference benchmark's protocol
+    (benchmark-mkl/matmul/bench_matmul.cpp:97-116).  Without the compiled reference: the plain-C
+    port on 4 images, one pass.  Also compares the GPU's output with the CPU's, bit for bit."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
-    from graph_oracle import run_graph
-    from oracle import Oracle
+    from graph_oracle import RefGraph, run_graph
+    from oracle import Oracle, Ref
     orc = Oracle()
     X = np.random.default_rng(5).standard_normal((32, 3, 224, 224)).astype(np.float32)
     y_gpu = model.run(X)
-    t0 = time.perf_counter()
-    y_cpu = run_graph(orc, payload, X[:sample])
-    dt = time.perf_counter() - t0
-    return {"samples_per_s": round(sample / dt, 2), "ms_per_image": round(dt / sample * 1e3, 1), "kind": "port",
-            "cores": orc.num_threads(), "sample": "%d of the 32 images, one pass" % sample,
-            "gpu_bit_exact_vs_cpu": bool(np.array_equal(y_cpu, y_gpu[:sample])),
-            "gpu_max_rel_err_vs_cpu": float(np.abs(y_cpu.astype(np.float64) - y_gpu[:sample]).max() / max(np.abs(y_cpu).max(), 1e-30))}
+    if Ref.available():
+        G = RefGraph(Ref(), orc, payload, (224, 224))
+        y_cpu, _ = G.run(X)
+        ts = [G.run(X)[1] for _ in range(3)]
+        G.close()
+        dt, n, kind = statistics.median(ts), 32, "reference"
+        sample = ("all 32 images, 1 warm-up + median of 3 passes, kernel time only; conv + FC layers: the reference's "
+                  "conv2d_rbm_fmajor_implicit / ellpack_matmul; max-pool, add, global average pool: plain-C port")
+    else:
+        n, kind, sample = 4, "port", "4 of the 32 images, one pass"
+        t0 = time.perf_counter()
+        y_cpu = run_graph(orc, payload, X[:n])
+        dt = time.perf_counter() - t0
+    return {"samples_per_s": round(n / dt, 2), "ms_per_image": round(dt / n * 1e3, 2), "kind": kind,
+            "cores": orc.num_threads(), "sample": sample, "avx512f": host_has_avx512f(),
+            "gpu_bit_exact_vs_cpu": bool(np.array_equal(y_cpu, y_gpu[:n])),
+            "gpu_max_rel_err_vs_cpu": float(np.abs(y_cpu.astype(np.float64) - y_gpu[:n]).max() / max(np.abs(y_cpu).max(), 1e-30))}
 
 
 def bench_cnn(steps, warmup, with_cpu=True):
@@ -353,6 +401,7 @@ def main():
     dX, dB, dY = ctx.array(X), ctx.array(bias), ctx.empty((E.m, C))
     step = lambda: ctx.matmul(dE, dX, C, dB, dY, "none")
     wall, ev_ms = time_launches(ctx, step, args.steps, args.warmup)
+    group_us = time_groups(ctx, step, 20, max(1, args.steps // 20))
     y_gpu = dY.download()
     # the row-per-wave kernel on the plain ROW layout, for comparison
     dE_row = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, hipabi.LAYOUT_ROW)
@@ -372,19 +421,24 @@ def main():
                    "m": E.m, "n": E.n, "r": E.r, "C": C, "sparsity": 0.9, "device": dev_name,
                    "spinup_ms": SPINUP_MS},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "ellpack_matmul_tiled_kernel", "kernel_us": round(ev_ms * 1e3, 2), "alg_bytes_per_launch": nbytes,
+                     "frac": round(gbps / HBM_PEAK_GBS, 4), "traffic": measured_traffic(HEADLINE_KERNEL),
+                     "kernel": HEADLINE_KERNEL, "kernel_us": round(ev_ms * 1e3, 2),
+                     # 20 event-bracketed groups of K/20 launches each, per launch
+                     "kernel_us_median": round(statistics.median(group_us), 2), "kernel_us_min": round(min(group_us), 2),
+                     "alg_bytes_per_launch": nbytes,
                      "row_kernel_us": round(ev_ms_row * 1e3, 2), "row_kernel_same_bits": row_bits_equal,
                      "valu_fp32_frac_of_157.3TF": round(flops / (ev_ms * 1e-3) / 1e12 / VALU_FP32_PEAK_TF, 4),
-                     "valu_fp32_frac_of_78.6TF_unpacked": round(flops / (ev_ms * 1e-3) / 1e12 / (VALU_FP32_PEAK_TF / 2), 4),
                      # every multiply-add needs a 4-byte X operand from LDS/L1 (no reuse in registers):
-                     # bytes at that level, and the fraction of what LDS can deliver (128 B/clk/CU)
+                     # bytes at that level, and the fraction of what LDS can deliver (256 B/clk/CU)
                      "gather_bytes": 8 * E.total_nnz + 4 * E.total_nnz * C + 4 * E.m * C,
-                     "lds_operand_frac_of_39.3TF": round(flops / (ev_ms * 1e-3) / 1e12 / LDS_OPERAND_PEAK_TF, 4),
+                     "lds_operand_frac_of_78.6TF": round(flops / (ev_ms * 1e-3) / 1e12 / LDS_OPERAND_PEAK_TF, 4),
                      "t_hbm_us": round(nbytes / (HBM_PEAK_GBS * 1e9) * 1e6, 2),
-                     "t_valu_us_unpacked": round(flops / (VALU_FP32_PEAK_TF / 2 * 1e12) * 1e6, 2),
-                     "t_bound_over_t": round(max(nbytes / (HBM_PEAK_GBS * 1e9), flops / (VALU_FP32_PEAK_TF / 2 * 1e12)) / (ev_ms * 1e-3), 4),
-                     "binding_bound": "operand delivery from LDS, then fp32 VALU issue (t_valu 10.9 us unpacked > t_hbm 2.7 us)"},
+                     "t_valu_us": round(flops / (VALU_FP32_PEAK_TF * 1e12) * 1e6, 2),
+                     "t_lds_operands_us": round(flops / (LDS_OPERAND_PEAK_TF * 1e12) * 1e6, 2),
+                     "t_bound_over_t": round(max(nbytes / (HBM_PEAK_GBS * 1e9), flops / (LDS_OPERAND_PEAK_TF * 1e12)) / (ev_ms * 1e-3), 4),
+                     "binding_bound": "not HBM (t_hbm 2.7 us): LDS operand reads (10.9 us at 256 B/clk/CU) and LDS tile writes (5.6 us at the "
+                                      "measured 78 B/clk/CU), multiply-adds in DPP form at half the plain rate (15 us with padding), and the "
+                                      "barrier between the 16 tile phases"},
     }
     if args.calibrate_copy:
         # A plain copy of known size (act_kernel<NONE>: reads N floats, writes N floats)

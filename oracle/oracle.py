@@ -259,6 +259,10 @@ class Ref:
         for nm in ("ref_relu_inplace", "ref_sigmoid_inplace", "ref_tanh_inplace"):
             getattr(L, nm).argtypes = [_f32p, ct.c_size_t]
         L.ref_conv.argtypes = [_f32p, _u32p, _f32p, ct.c_int, ct.c_int, _f32p, ct.c_uint32, _f32p]
+        L.ref_conv_plan.restype = ct.c_void_p
+        L.ref_conv_plan.argtypes = [_f32p, _u32p, _f32p, ct.c_int, ct.c_int]
+        L.ref_conv_run.argtypes = [ct.c_void_p, _f32p, ct.c_uint32, _f32p]
+        L.ref_conv_plan_free.argtypes = [ct.c_void_p]
         L.ref_rbm_sizes.argtypes = [ct.c_void_p, ct.c_uint32, _u32p]
         L.ref_rbm_copy.argtypes = [ct.c_void_p, ct.c_uint32, _u32p, _u32p, _u32p, ct.POINTER(ct.c_uint16), _f32p]
 
@@ -336,3 +340,19 @@ class Ref:
         dst = np.empty(g.Cout * g.H_out * g.W_out * B, dtype=np.float32)
         self.lib.ref_conv(_fp(Wdense), _up(geom), _fp(bias), int(fuse_relu), variant, _fp(src), B, _fp(dst))
         return dst
+
+    def conv_plan(self, Wdense, g, bias=None, fuse_relu=False, variant=0):
+        """The load-time part of a convolution layer (encode, kmap, RBM plan) -> a handle for conv_run."""
+        Wdense = _f32(Wdense)
+        bias = None if bias is None else _f32(bias)
+        geom = np.array([getattr(g, k) for k, _ in ConvGeom._fields_], dtype=np.uint32)
+        return self.lib.ref_conv_plan(_fp(Wdense), _up(geom), _fp(bias), int(fuse_relu), variant)
+
+    def conv_run(self, plan, g, src, B, out=None):
+        src = _f32(src)
+        dst = out if out is not None else np.empty(g.Cout * g.H_out * g.W_out * B, dtype=np.float32)
+        self.lib.ref_conv_run(plan, _fp(src), B, _fp(dst))
+        return dst
+
+    def conv_plan_free(self, plan):
+        self.lib.ref_conv_plan_free(plan)

@@ -18,6 +18,7 @@
 #include <cstdint>
 #include <cstring>
 #include <utility>
+#include <vector>
 
 #include "ellpack_encoder.hpp"
 #include "ellpack_matmul.hpp"
@@ -96,11 +97,20 @@ void ref_tanh_inplace(float *d, size_t n) { tanh_inplace(d, n); }
 // The ConvAttr is filled the way the reference's loader fills it
 // (src/sparse_onnx.cpp:394-502): weights Cout x K row-major, kmap in (cin,kh,kw)
 // order with dh = kh*dil - pad, patch_indices with a one-past sentinel.
-void ref_conv(const float *Wdense, const uint32_t *geom, const float *bias, int fuse_relu,
-              int variant, const float *src, uint32_t B, float *dst)
+struct RefConvPlan {
+    ConvAttr attr;
+    std::vector<float> bias;
+    int variant;
+};
+
+// Load-time part (what the reference's loader does once per layer): encode, kmap, patch_indices
+// (variant 1), RBM plan (variant 3).  The bias is copied.
+void *ref_conv_plan(const float *Wdense, const uint32_t *geom, const float *bias, int fuse_relu, int variant)
 {
-    ConvAttr c{convert_to_ellpack(Wdense, geom[1], geom[0] * geom[2] * geom[3])};
-    c.bias_ptr = const_cast<float *>(bias);
+    auto *p = new RefConvPlan{ConvAttr{convert_to_ellpack(Wdense, geom[1], geom[0] * geom[2] * geom[3])}, {}, variant};
+    ConvAttr &c = p->attr;
+    if (bias) p->bias.assign(bias, bias + geom[1]);
+    c.bias_ptr = bias ? p->bias.data() : nullptr;
     c.Cin = geom[0]; c.Cout = geom[1]; c.kH = geom[2]; c.kW = geom[3];
     c.stride_h = geom[4]; c.stride_w = geom[5];
     c.pad_h = geom[6]; c.pad_w = geom[7];
@@ -128,16 +138,33 @@ void ref_conv(const float *Wdense, const uint32_t *geom, const float *bias, int 
                 }
     }
     if (variant == 3) {
-        c.rbm = build_rbm_from_ellpack(c.E, bias, 8);
+        c.rbm = build_rbm_from_ellpack(c.E, c.bias_ptr, 8);
         c.use_rbm = true;
     }
-    switch (variant) {
-    case 0: conv2d_patchmajor_tiled(c, src, B, dst); break;
-    case 1: conv2d_tiled_im2col_fmajor(c, src, B, dst); break;
-    case 2: conv2d_tiled_im2col_cmajor(c, src, B, dst); break;
-    case 3: conv2d_rbm_fmajor_implicit(c, src, B, dst); break;
+    return p;
+}
+
+// The per-call part: one of the reference's convolution kernels on a prepared layer.
+void ref_conv_run(void *plan, const float *src, uint32_t B, float *dst)
+{
+    const RefConvPlan *p = static_cast<RefConvPlan *>(plan);
+    switch (p->variant) {
+    case 0: conv2d_patchmajor_tiled(p->attr, src, B, dst); break;
+    case 1: conv2d_tiled_im2col_fmajor(p->attr, src, B, dst); break;
+    case 2: conv2d_tiled_im2col_cmajor(p->attr, src, B, dst); break;
+    case 3: conv2d_rbm_fmajor_implicit(p->attr, src, B, dst); break;
     default: break;
     }
+}
+
+void ref_conv_plan_free(void *plan) { delete static_cast<RefConvPlan *>(plan); }
+
+void ref_conv(const float *Wdense, const uint32_t *geom, const float *bias, int fuse_relu,
+              int variant, const float *src, uint32_t B, float *dst)
+{
+    void *p = ref_conv_plan(Wdense, geom, bias, fuse_relu, variant);
+    ref_conv_run(p, src, B, dst);
+    ref_conv_plan_free(p);
 }
 
 // build_rbm_from_ellpack on the handle's matrix, flattened: sizes = {blocks, union columns, pairs};

@@ -1,0 +1,177 @@
+"""Condenses rocprofv3 output into the short text summaries kept under profiles/.
+
+    # counters (one rocprofv3 --pmc run per counter group; csv output):
+    python sparse-ops_amd/bench/pmc_summary.py counters <counter_collection.csv> [...more csv] [--kernels REGEX]
+    # kernel durations of a --kernel-trace run (csv output):
+    python sparse-ops_amd/bench/pmc_summary.py trace <kernel_trace.csv> [--kernels REGEX] [--skip N]
+    # HBM-side bytes per launch from a FETCH_SIZE run and a WRITE_SIZE run, scaled by the plain copy
+    # kernel of known size that `bench.py --calibrate-copy` launches, written into the table bench.py
+    # reads `roofline.traffic` from:
+    python sparse-ops_amd/bench/pmc_summary.py traffic <fetch.csv> <write.csv> --update profiles/hbm_traffic.json
+
+Every mode prints per-kernel averages per dispatch; template arguments are kept, argument lists cut.
+"""
+import argparse
+import collections
+import csv
+import hashlib
+import json
+import os
+import re
+import statistics
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+COPY_KERNEL = "act_kernel<0>"
+COPY_KIB = 262144.0      # bench.py --calibrate-copy: 256 MiB read, 256 MiB written per launch
+
+# Source files whose text decides a kernel's memory traffic: the table stores their hash, and
+# bench.py reports a kernel's traffic only while the hash still matches.
+KERNEL_SOURCES = {
+    "ellpack_matmul_tiled_kernel": ["sparse-ops_amd/csrc/matmul_tiled.hip", "sparse-ops_amd/csrc/dpp_steps.h",
+                                    "sparse-ops_amd/csrc/so_internal.h"],
+    "ellpack_matmul_kernel": ["sparse-ops_amd/csrc/matmul.hip", "sparse-ops_amd/csrc/so_internal.h"],
+    "matvec_rows_kernel": ["sparse-ops_amd/csrc/matvec.hip"],
+    "matvec_binned_kernel": ["sparse-ops_amd/csrc/matvec.hip"],
+}
+
+
+def short_name(name):
+    """void ns::kernel<1, 2>(args...) [clone] -> kernel<1, 2>"""
+    name = re.sub(r"\s*\[clone.*$", "", name.strip())
+    name = name.replace("(anonymous namespace)::", "")
+    depth, cut = 0, len(name)
+    for i, ch in enumerate(name):
+        if ch == "<":
+            depth += 1
+        elif ch == ">":
+            depth -= 1
+        elif ch == "(" and depth == 0:
+            cut = i
+            break
+    return re.sub(r"^void\s+", "", name[:cut]).replace(", ", ",")
+
+
+def source_hash(kernel):
+    """sha1 over the kernel's source files (None for a kernel not in KERNEL_SOURCES)."""
+    base = kernel.split("<")[0]
+    files = KERNEL_SOURCES.get(base)
+    if not files:
+        return None
+    h = hashlib.sha1()
+    for f in files:
+        with open(os.path.join(ROOT, f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
+def read_counters(paths, pattern):
+    vals = collections.defaultdict(lambda: collections.defaultdict(list))
+    for path in paths:
+        with open(path, newline="") as f:
+            for r in csv.DictReader(f):
+                k = short_name(r["Kernel_Name"])
+                if pattern and not re.search(pattern, k):
+                    continue
+                vals[k][r["Counter_Name"]].append(float(r["Counter_Value"]))
+    return vals
+
+
+def cmd_counters(a):
+    vals = read_counters(a.csv, a.kernels)
+    print("%-52s %-28s %10s %18s %16s %16s" % ("kernel", "counter", "dispatches", "avg per dispatch", "min", "max"))
+    for k in sorted(vals):
+        for c in sorted(vals[k]):
+            v = vals[k][c]
+            print("%-52s %-28s %10d %18.1f %16.1f %16.1f" % (k, c, len(v), sum(v) / len(v), min(v), max(v)))
+
+
+def cmd_trace(a):
+    dur = collections.defaultdict(list)
+    with open(a.csv[0], newline="") as f:
+        for r in csv.DictReader(f):
+            k = short_name(r["Kernel_Name"])
+            if a.kernels and not re.search(a.kernels, k):
+                continue
+            dur[k].append((int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3)
+    total = sum(sum(v) for v in dur.values())
+    print("%-52s %8s %12s %12s %12s %12s %8s" % ("kernel", "calls", "avg us", "median us", "min us", "max us", "% time"))
+    for k, v in sorted(dur.items(), key=lambda kv: -sum(kv[1])):
+        w = v[a.skip:] if len(v) > a.skip else v
+        print("%-52s %8d %12.2f %12.2f %12.2f %12.2f %8.1f" % (k, len(v), sum(w) / len(w), statistics.median(w), min(w), max(w),
+                                                               100.0 * sum(v) / total))
+    if a.skip:
+        print("(avg / median / min / max leave out each kernel's first %d calls)" % a.skip)
+
+
+def cmd_traffic(a):
+    fetch = read_counters([a.csv[0]], None)
+    write = read_counters([a.csv[1]], None)
+
+    def avg(table, kernel, counter):
+        v = table.get(kernel, {}).get(counter)
+        return sum(v) / len(v) if v else None
+    f_copy, w_copy = avg(fetch, COPY_KERNEL, "FETCH_SIZE"), avg(write, COPY_KERNEL, "WRITE_SIZE")
+    if not f_copy or not w_copy:
+        sys.exit("the runs hold no %s dispatches: run bench.py with --calibrate-copy" % COPY_KERNEL)
+    f_scale, w_scale = COPY_KIB / f_copy, COPY_KIB / w_copy
+    print("calibration: %s reads and writes %.0f KiB; FETCH_SIZE reads %.1f (x %.3f), WRITE_SIZE reads %.1f (x %.3f)"
+          % (COPY_KERNEL, COPY_KIB, f_copy, f_scale, w_copy, w_scale))
+    table = {}
+    if a.update and os.path.exists(a.update):
+        with open(a.update) as f:
+            table = json.load(f)
+    print("%-52s %14s %14s %16s" % ("kernel", "fetched KiB", "written KiB", "bytes per launch"))
+    for k in sorted(fetch):
+        if k == COPY_KERNEL or k.startswith("__amd") or (a.kernels and not re.search(a.kernels, k)):
+            continue
+        fk, wk = avg(fetch, k, "FETCH_SIZE"), avg(write, k, "WRITE_SIZE")
+        if fk is None or wk is None:
+            continue
+        nbytes = int(round((fk * f_scale + wk * w_scale) * 1024))
+        print("%-52s %14.1f %14.1f %16d" % (k, fk * f_scale, wk * w_scale, nbytes))
+        sha = source_hash(k)
+        if sha:
+            entry = {"bytes_per_launch": nbytes, "fetched_kib": round(fk * f_scale, 1), "written_kib": round(wk * w_scale, 1),
+                     "fetch_scale": round(f_scale, 4), "write_scale": round(w_scale, 4), "source_sha1": sha,
+                     "dispatches": len(fetch[k]["FETCH_SIZE"])}
+            if a.workload:
+                entry["workload"] = a.workload
+            table[k if not a.workload else k + " | " + a.workload] = entry
+    if a.update:
+        with open(a.update, "w") as f:
+            json.dump(table, f, indent=1, sort_keys=True)
+            f.write("\n")
+        print("updated", a.update)
+
+
+def lookup_traffic(table_path, kernel, workload=None):
+    """bench.py's reader: bytes per launch of `kernel` (with its template arguments, or the bare name:
+    then any instantiation measured on `workload` matches), or None when the table has no such entry
+    or the kernel's sources have changed since it was measured."""
+    try:
+        with open(table_path) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None
+    for key, e in table.items():
+        name, _, wl = key.partition(" | ")
+        if (name == kernel or name.split("<")[0] == kernel) and (workload is None or wl == workload):
+            return e["bytes_per_launch"] if e.get("source_sha1") == source_hash(name) else None
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("mode", choices=["counters", "trace", "traffic"])
+    ap.add_argument("csv", nargs="+")
+    ap.add_argument("--kernels", default=None, help="regular expression on the short kernel name")
+    ap.add_argument("--skip", type=int, default=0, help="trace: calls to leave out of the averages (warm-up)")
+    ap.add_argument("--update", default=None, help="traffic: JSON table to update")
+    ap.add_argument("--workload", default=None, help="traffic: key suffix when one kernel is measured on several workloads")
+    a = ap.parse_args()
+    {"counters": cmd_counters, "trace": cmd_trace, "traffic": cmd_traffic}[a.mode](a)
+
+
+if __name__ == "__main__":
+    main()
