@@ -260,7 +260,7 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
     // this lane's output pixel and its corner inside the window
     const uint32_t pl = pgi * PPW + lane / LPP, b4 = lane % LPP;
     const bool pvalid = pl < a.TH * a.TW;
-    const uint32_t pc = pvalid ? pl : 0u;
+    const uint32_t pc = pvalid ? window_slot_pixel(a, pl) : 0u;
     const uint32_t ty = pc / a.TW, tx = pc % a.TW;
     const bool live = computes && pvalid && th0 + ty < g.H_out && tw0 + tx < g.W_out;
     const uint32_t lanebase = ((ty * a.sth * a.IW + tx * a.stw) << SHIFT) + b4 * 16u;   // bytes
@@ -490,6 +490,7 @@ so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, 
     a.nbuf = w.nch > 1 ? 2u : 1u;
     a.sth = window_step(plan->g.kH, plan->g.stride_h); a.stw = window_step(plan->g.kW, plan->g.stride_w);
     a.sbh = window_subsample(plan->g.kH, plan->g.stride_h); a.sbw = window_subsample(plan->g.kW, plan->g.stride_w);
+    window_pixel_order(a, LPP);
     const size_t lds = (size_t)a.nbuf * a.buf_f4 * 16;
     // a layout whose chunks were sized for a smaller batch tile than this batch's does not fit
     if (LPP > w.lpp && (lds > (size_t)ctx->max_lds_bytes || a.win_f4 > (uint32_t)kWinMaxPerThread * kWinThreads)) return SO_OK;
@@ -581,7 +582,7 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     const uint32_t lpp_for_batch = window_lpp(batch) ? window_lpp(batch) : kWinLPP;
     uint32_t max_px = (uint64_t)g.H_out * g.W_out <= 256 ? 16u : 32u;
     if (lpp_for_batch < kWinLPP) max_px = 64u / lpp_for_batch;
-    if (ctx->tune.conv_tilepx > 0) max_px = (uint32_t)ctx->tune.conv_tilepx;
+    if (ctx->tune.conv_tilepx > 0) max_px = std::min(64u, (uint32_t)ctx->tune.conv_tilepx);   // the slot table holds 64 pixels
     for (uint32_t th = 1; th <= max_px && th <= g.H_out; ++th)
         for (uint32_t tw = 1; th * tw <= max_px && tw <= g.W_out; ++tw) {
             const uint64_t tiles = (uint64_t)so_ceil_div(g.H_out, th) * so_ceil_div(g.W_out, tw);

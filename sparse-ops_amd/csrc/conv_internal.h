@@ -3,6 +3,9 @@
 
 #include "so_internal.h"
 
+#include <algorithm>
+#include <vector>
+
 // What the LDS-windowed kernel needs on top of the plan; built only for geometries it suits.
 // The input channels are cut into chunks of `cc`; for one chunk and one tile of TH x TW output
 // pixels the input window is IH x IW pixels.  A stored nonzero becomes the entry {weight bits,
@@ -64,6 +67,7 @@ struct WinArgs {
     uint32_t nbuf;      // 2: double-buffered windows; 1: a single chunk, nothing to overlap
     uint32_t sth, stw;  // window pixels between neighbouring output pixels
     uint32_t sbh, sbw;  // input pixels between neighbouring window pixels
+    uint32_t order[16]; // slot -> output pixel of the tile (ty * TW + tx), one byte per slot; see window_pixel_order
 };
 
 // Along an axis on which the kernel has a single tap, a strided convolution reads only every
@@ -72,3 +76,51 @@ struct WinArgs {
 inline uint32_t window_step(uint32_t k, uint32_t stride) { return k == 1 ? 1u : stride; }
 inline uint32_t window_subsample(uint32_t k, uint32_t stride) { return k == 1 ? stride : 1u; }
 
+// Which output pixel of the tile each pixel slot of the workgroup computes (slot = lanes / lanes per
+// pixel, wave after wave).  LDS serves a 16-byte read 16 lanes at a time: 16 / lpp pixels, each a run
+// of 16 * lpp bytes at (window pixel index) * 16 * lpp, i.e. on the bank group (window pixel index)
+// mod (16 / lpp).  Pixels taken in row-major order collide on a bank group whenever the tile's rows
+// are not a multiple of 16 / lpp pixels wide (tiles 7 pixels wide: every second read takes two
+// turns).  Which slot computes which pixel is free, so the slots are dealt out such that the
+// pixels of each group of 16 / lpp slots fall on different bank groups wherever the tile's shape
+// allows it.  At most 64 pixels per tile.
+inline void window_pixel_order(WinArgs &a, uint32_t lpp)
+{
+    const uint32_t m = 16u / lpp, npx = a.TH * a.TW;
+    std::vector<std::vector<uint8_t>> bucket(m);
+    for (uint32_t p = 0; p < npx && p < 64u; ++p)
+        bucket[((p / a.TW) * a.sth * a.IW + (p % a.TW) * a.stw) % m].push_back((uint8_t)p);
+    for (auto &b : bucket) std::reverse(b.begin(), b.end());       // pop_back hands out the lowest pixel first
+    uint8_t slots[64] = {0};
+    uint32_t filled = 0;
+    while (filled < npx && filled < 64u) {
+        // one group: a pixel from each bank group, fullest first; then, if some are exhausted, more from the fullest
+        std::vector<uint32_t> by_size(m);
+        for (uint32_t r = 0; r < m; ++r) by_size[r] = r;
+        std::stable_sort(by_size.begin(), by_size.end(), [&](uint32_t x, uint32_t y) { return bucket[x].size() > bucket[y].size(); });
+        uint32_t taken = 0;
+        for (uint32_t pass = 0; taken < m && filled < npx && filled < 64u; ++pass) {
+            bool any = false;
+            for (uint32_t k = 0; k < m && taken < m && filled < npx && filled < 64u; ++k) {
+                std::vector<uint8_t> &b = bucket[by_size[k]];
+                if (b.empty()) continue;
+                slots[filled++] = b.back();
+                b.pop_back();
+                ++taken;
+                any = true;
+            }
+            if (!any) break;
+        }
+    }
+    for (uint32_t i = 0; i < 16; ++i)
+        a.order[i] = (uint32_t)slots[4 * i] | ((uint32_t)slots[4 * i + 1] << 8) | ((uint32_t)slots[4 * i + 2] << 16) | ((uint32_t)slots[4 * i + 3] << 24);
+}
+
+// The kernels' side: the output pixel of slot `pl` (< 64).
+__device__ __forceinline__ uint32_t window_slot_pixel(const WinArgs &a, uint32_t pl)
+{
+    uint32_t word = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < 16; ++i) word = (pl >> 2) == i ? a.order[i] : word;
+    return (word >> ((pl & 3u) * 8u)) & 0xffu;
+}

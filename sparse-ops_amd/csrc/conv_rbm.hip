@@ -212,7 +212,7 @@ void conv2d_rbm_kernel(const int4 *__restrict__ sets, const uint32_t *__restrict
     // this lane's output pixel and its corner inside the window
     const uint32_t pl = pgi * PPW + lane / LPP, b4 = lane % LPP;
     const bool pvalid = pl < a.TH * a.TW;
-    const uint32_t pc = pvalid ? pl : 0u;
+    const uint32_t pc = pvalid ? window_slot_pixel(a, pl) : 0u;
     const uint32_t ty = pc / a.TW, tx = pc % a.TW;
     const bool live = computes && pvalid && th0 + ty < g.H_out && tw0 + tx < g.W_out;
     const uint32_t lanebase = ((ty * a.sth * a.IW + tx * a.stw) << SHIFT) + b4 * 16u;   // bytes
@@ -507,6 +507,7 @@ so_status so_conv_rbm_launch(so_ctx *ctx, const so_conv_plan *plan, const float 
     a.nbuf = w.nch > 1 ? 2u : 1u;
     a.sth = window_step(plan->g.kH, plan->g.stride_h); a.stw = window_step(plan->g.kW, plan->g.stride_w);
     a.sbh = window_subsample(plan->g.kH, plan->g.stride_h); a.sbw = window_subsample(plan->g.kW, plan->g.stride_w);
+    window_pixel_order(a, LPP);
     const size_t lds = (size_t)a.nbuf * a.buf_f4 * 16;
     // a layout whose chunks were sized for a smaller batch tile than this batch's does not fit
     if (LPP > w.lpp && (lds > (size_t)ctx->max_lds_bytes || a.win_f4 > (uint32_t)kRbmMaxPerThread * kWinThreads)) return SO_OK;
