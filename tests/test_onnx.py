@@ -248,3 +248,24 @@ def test_mutated_model_files_raise_cleanly(backend, tmp_path, name):
         except RuntimeError:
             pass
     assert loaded < 80
+
+
+def test_loader_under_sanitizers(tmp_path):
+    """The host ONNX loader, built with AddressSanitizer + UndefinedBehaviorSanitizer
+    (`make -C sparse-ops_amd asan`, tests/cpp/fuzz_onnx.cpp), on 2000 mutations of the four
+    torch-exported models: truncations, flipped bytes, oversized varints, repeated slices.  Every
+    file must end in a loaded model or an exception; any sanitizer report fails the run."""
+    import glob
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    binary = os.path.join(root, "tests", "cpp", "fuzz_onnx_asan")
+    if not os.path.exists(binary):
+        subprocess.run(["make", "-C", os.path.join(root, "sparse-ops_amd"), "asan"], check=True, stdout=subprocess.DEVNULL)
+    models = sorted(glob.glob(os.path.join(root, "tests", "golden", "torch_export", "*.onnx")))
+    assert len(models) == 4
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
+    out = subprocess.run([binary, "500", str(tmp_path)] + models, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                         errors="replace", env=env, timeout=300)        # messages quote mutated names: any bytes
+    assert out.returncode == 0, out.stdout[-4000:]
+    assert "2000 mutated files, no crash" in out.stdout
+    assert "AddressSanitizer" not in out.stdout and "runtime error" not in out.stdout, out.stdout[-4000:]
