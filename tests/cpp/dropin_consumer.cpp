@@ -1,10 +1,12 @@
 // A C++ caller written against the reference's headers only (ellpack_encoder.hpp,
-// ellpack_matmul.hpp, ellpack_matvec.hpp, sparse_onnx.hpp): host pointers in, host pointers out,
+// ellpack_matmul.hpp, ellpack_matvec.hpp, activations.hpp, conv_kernels.hpp, rbm_conv.hpp, sparse_onnx.hpp): host pointers in, host pointers out,
 // as benchmark-mkl/matmul/bench_matmul.cpp:98 and benchmark-mkl/matvec/bench_matvec.cpp:100 of the
 // reference call them.  Checks every result against plain loops and exits non-zero on a mismatch.
 //
 //   dropin_consumer                      kernels only
 //   dropin_consumer model.onnx in.bin expected.bin B     + SparseOnnxModel::run, bit for bit
+#include "activations.hpp"
+#include "conv_kernels.hpp"
 #include "ellpack_encoder.hpp"
 #include "ellpack_matmul.hpp"
 #include "ellpack_matvec.hpp"
@@ -113,6 +115,94 @@ int main(int argc, char **argv)
         for (uint32_t c : E.nnz) stored += c;
         check(ordered && pairs == stored && std::memcmp(again.data(), W.data(), again.size() * sizeof(float)) == 0,
               "build_rbm_from_ellpack: ordered, complete, decodes to W");
+    }
+
+    // activations.hpp (include/activations.hpp:10-16 of the reference): in place over a host buffer
+    {
+        std::vector<float> a(1000), r, sg, th;
+        for (auto &v : a) v = 3.0f * gauss(rng);
+        r = sg = th = a;
+        relu_inplace(r.data(), r.size());
+        sigmoid_inplace(sg.data(), sg.size());
+        tanh_inplace(th.data(), th.size());
+        bool ok = true;
+        for (size_t i = 0; i < a.size(); ++i) {
+            ok &= r[i] == (a[i] > 0.0f ? a[i] : 0.0f);
+            ok &= std::fabs(sg[i] - 1.0f / (1.0f + std::exp(-a[i]))) <= 1e-6f;
+            ok &= std::fabs(th[i] - std::tanh(a[i])) <= 1e-6f;
+        }
+        check(ok, "relu_inplace exact, sigmoid_inplace / tanh_inplace within 1e-6");
+    }
+
+    // conv_kernels.hpp (include/conv_kernels.hpp:8-36): the four entry points on their three layouts against
+    // the direct definition (src/layers/conv.cpp:44-107: bias, then one fmaf per stored tap in slot order,
+    // taps outside the image skipped)
+    {
+        const uint32_t Cin = 5, Cout = 40, kH = 3, kW = 3, H = 9, Wd_ = 11, B = 8, sh = 2, sw = 1, ph = 1, pw = 1;
+        const uint32_t Ho = (H + 2 * ph - kH) / sh + 1, Wo = (Wd_ + 2 * pw - kW) / sw + 1, K = Cin * kH * kW;
+        std::vector<float> Wc(size_t(Cout) * K), cb(Cout), src(size_t(Cin) * H * Wd_ * B);
+        for (auto &v : Wc) v = coin(rng) < 0.6f ? 0.0f : gauss(rng);
+        for (auto &v : cb) v = gauss(rng);
+        for (auto &v : src) v = gauss(rng);
+        ConvAttr c{convert_to_ellpack(Wc.data(), Cout, K)};
+        c.bias_ptr = cb.data();
+        c.Cin = Cin; c.Cout = Cout; c.kH = kH; c.kW = kW; c.stride_h = sh; c.stride_w = sw; c.pad_h = ph; c.pad_w = pw;
+        c.H_in = H; c.W_in = Wd_; c.H_out = Ho; c.W_out = Wo;
+        c.fuse_relu = true;
+        std::vector<float> ref(size_t(Cout) * Ho * Wo * B);         // [C][H][W][B]
+        for (uint32_t co = 0; co < Cout; ++co)
+            for (uint32_t ho = 0; ho < Ho; ++ho)
+                for (uint32_t wo = 0; wo < Wo; ++wo)
+                    for (uint32_t b = 0; b < B; ++b) {
+                        float acc = cb[co];
+                        for (uint32_t s2 = 0; s2 < c.E.nnz[co]; ++s2) {
+                            const uint32_t k = c.E.idx[size_t(co) * c.E.r + s2], ci = k / (kH * kW), kh = (k / kW) % kH, kw = k % kW;
+                            const int hi = int(ho * sh + kh) - int(ph), wi = int(wo * sw + kw) - int(pw);
+                            if (hi < 0 || wi < 0 || hi >= int(H) || wi >= int(Wd_)) continue;
+                            acc = std::fmaf(c.E.Wd.ptr[size_t(co) * c.E.r + s2], src[((size_t(ci) * H + hi) * Wd_ + wi) * B + b], acc);
+                        }
+                        ref[((size_t(co) * Ho + ho) * Wo + wo) * B + b] = acc > 0.0f ? acc : 0.0f;
+                    }
+        std::vector<float> out(ref.size(), NAN);
+        conv2d_patchmajor_tiled(c, src.data(), B, out.data());
+        check(std::memcmp(out.data(), ref.data(), out.size() * sizeof(float)) == 0, "conv2d_patchmajor_tiled bit-exact");
+        c.rbm = build_rbm_from_ellpack(c.E, cb.data());
+        c.use_rbm = true;
+        std::fill(out.begin(), out.end(), NAN);
+        conv2d_patchmajor_tiled(c, src.data(), B, out.data());
+        check(std::memcmp(out.data(), ref.data(), out.size() * sizeof(float)) == 0, "conv2d_patchmajor_tiled with the RBM plan attached");
+        // the same tensors in the Fortran (B,C,H,W) and the C-order (B,C,H,W) layouts
+        std::vector<float> srcF(src.size()), srcC(src.size()), outF(ref.size(), NAN), outC(ref.size(), NAN);
+        for (uint32_t ci = 0; ci < Cin; ++ci)
+            for (uint32_t h = 0; h < H; ++h)
+                for (uint32_t w = 0; w < Wd_; ++w)
+                    for (uint32_t b = 0; b < B; ++b) {
+                        const float v = src[((size_t(ci) * H + h) * Wd_ + w) * B + b];
+                        srcF[b + size_t(B) * (ci + size_t(Cin) * (h + size_t(H) * w))] = v;
+                        srcC[((size_t(b) * Cin + ci) * H + h) * Wd_ + w] = v;
+                    }
+        conv2d_rbm_fmajor_implicit(c, srcF.data(), B, outF.data());
+        conv2d_tiled_im2col_cmajor(c, srcC.data(), B, outC.data());
+        bool okF = true, okC = true;
+        for (uint32_t co = 0; co < Cout; ++co)
+            for (uint32_t h = 0; h < Ho; ++h)
+                for (uint32_t w = 0; w < Wo; ++w)
+                    for (uint32_t b = 0; b < B; ++b) {
+                        const float v = ref[((size_t(co) * Ho + h) * Wo + w) * B + b];
+                        okF &= outF[b + size_t(B) * (co + size_t(Cout) * (h + size_t(Ho) * w))] == v;
+                        okC &= outC[((size_t(b) * Cout + co) * Ho + h) * Wo + w] == v;
+                    }
+        check(okF, "conv2d_rbm_fmajor_implicit (Fortran layout) bit-exact");
+        std::fill(outF.begin(), outF.end(), NAN);
+        conv2d_tiled_im2col_fmajor(c, srcF.data(), B, outF.data());
+        bool okF2 = true;
+        for (uint32_t co = 0; co < Cout; ++co)
+            for (uint32_t h = 0; h < Ho; ++h)
+                for (uint32_t w = 0; w < Wo; ++w)
+                    for (uint32_t b = 0; b < B; ++b)
+                        okF2 &= outF[b + size_t(B) * (co + size_t(Cout) * (h + size_t(Ho) * w))] == ref[((size_t(co) * Ho + h) * Wo + w) * B + b];
+        check(okF2, "conv2d_tiled_im2col_fmajor bit-exact");
+        check(okC, "conv2d_tiled_im2col_cmajor (C-order layout) bit-exact");
     }
 
     if (argc == 5) {
