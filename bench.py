@@ -379,6 +379,9 @@ def main():
                     help="untimed launches of each measured kernel for this long before its warm-up steps (clock settling)")
     ap.add_argument("--no-extras", action="store_true", help="skip matvec and MLP measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
+    ap.add_argument("--skip-extra", action="append", default=[], metavar="NAME",
+                    help="leave out one entry of `extras` (e.g. matvec_uniform_65536_rows, which runs the same kernel as "
+                         "matvec_uniform: counter passes that average per kernel name need the two apart); repeatable")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain 256 MiB copy kernel (scale factor for rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -488,11 +491,12 @@ def main():
         extras["matvec_zipf"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048",
                                              datagen.config2b, hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS, hipabi.LAYOUT_BINS,
                                              k, args.warmup, not args.no_cpu)
-        log("matvec 65536x16384 uniform ...")
-        # four times the rows of config 2a: what the same kernel streams once its fixed per-launch cost is amortised
-        extras["matvec_uniform_65536_rows"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 65536x16384, 95% Bernoulli",
-                                                           lambda: datagen.uniform_ellpack(48, 65536, 16384, 0.05),
-                                                           hipabi.LAYOUT_ROW, hipabi.LAYOUT_ROW, max(10, k // 4), 3, False)
+        if "matvec_uniform_65536_rows" not in args.skip_extra:
+            log("matvec 65536x16384 uniform ...")
+            # four times the rows of config 2a: what the same kernel streams once its fixed per-launch cost is amortised
+            extras["matvec_uniform_65536_rows"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 65536x16384, 95% Bernoulli",
+                                                               lambda: datagen.uniform_ellpack(48, 65536, 16384, 0.05),
+                                                               hipabi.LAYOUT_ROW, hipabi.LAYOUT_ROW, max(10, k // 4), 3, False)
         log("sparse MLP ...")
         extras["mlp"] = bench_mlp(k, args.warmup, with_cpu=not args.no_cpu)
         log("sparse CNN ...")
