@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 
 #include "dpp_steps.h"
+#include "conv_internal.h"
 
 #include <algorithm>
 #include <cstdint>
@@ -84,6 +85,7 @@ __device__ __forceinline__ void steps8_v3(const char *lds, uint32_t base, u32x2 
 //             each lane its own 16 / 8 / 4 bytes (consecutive lanes, consecutive addresses: no bank
 //             conflict), results never used.
 // MODE 18:    8 ds_write_b128 per iteration.
+// MODE 19:    8 ds_read_b128 per iteration, every lane at an address of its own (bank-conflict patterns).
 // MODE 3:     32 independent v_fma_f32 per iteration, no memory access.
 // MODE 4:     32 v_fmac_f32_dpp row_newbcast per iteration (the multiply-add of the LDS-fed kernels' steps).
 // MODE 5:     the step loop of the tiled matmul and the windowed convolution itself (csrc/dpp_steps.h):
@@ -132,6 +134,13 @@ __global__ __launch_bounds__(kThreads) void probe(float *out, unsigned long long
                          "ds_read_b32 %3, %8 offset:768\n\tds_read_b32 %4, %8\n\tds_read_b32 %5, %8 offset:256\n\t"
                          "ds_read_b32 %6, %8 offset:512\n\tds_read_b32 %7, %8 offset:768\n\ts_waitcnt lgkmcnt(0)"
                          : "=&v"(x0), "=&v"(x1), "=&v"(x2), "=&v"(x3), "=&v"(x4), "=&v"(x5), "=&v"(x6), "=&v"(x7) : "v"(addr));
+        } else if constexpr (MODE == 19) {
+            // ds_read_b128 with this lane's address taken from a table: which lane groups share a turn of the banks
+            f32x4 x0, x1, x2, x3, x4, x5, x6, x7;
+            asm volatile("ds_read_b128 %0, %8\n\tds_read_b128 %1, %8 offset:16384\n\tds_read_b128 %2, %8 offset:32768\n\t"
+                         "ds_read_b128 %3, %8 offset:49152\n\tds_read_b128 %4, %8\n\tds_read_b128 %5, %8 offset:16384\n\t"
+                         "ds_read_b128 %6, %8 offset:32768\n\tds_read_b128 %7, %8 offset:49152\n\ts_waitcnt lgkmcnt(0)"
+                         : "=&v"(x0), "=&v"(x1), "=&v"(x2), "=&v"(x3), "=&v"(x4), "=&v"(x5), "=&v"(x6), "=&v"(x7) : "v"(eo));
         } else if constexpr (MODE == 18) {
             f32x4 v = {1.f, 2.f, 3.f, (float)it};
             asm volatile("ds_write_b128 %0, %1\n\tds_write_b128 %0, %1 offset:1024\n\tds_write_b128 %0, %1 offset:2048\n\t"
@@ -276,6 +285,53 @@ int main()
     float *dEnts;
     CK(hipMalloc(&dEnts, ents.size() * 4));
     CK(hipMemcpy(dEnts, ents.data(), ents.size() * 4, hipMemcpyHostToDevice));
+    // ds_read_b128 address patterns (byte address of each lane inside a 16 KB region)
+    {
+        struct { const char *what; uint32_t (*addr)(uint32_t); } pats[] = {
+            {"64 lanes x 16 B contiguous", [](uint32_t l) { return l * 16u; }},
+            {"4 groups of 16 lanes, each 256 B contiguous, all on the same banks", [](uint32_t l) { return (l % 16u) * 16u + (l / 16u) * 4096u; }},
+            {"8 groups of 8 lanes, each 128 B contiguous, all on banks 0-31", [](uint32_t l) { return (l % 8u) * 16u + (l / 8u) * 2048u; }},
+            {"8 groups of 8 lanes, odd groups on banks 32-63", [](uint32_t l) { return (l % 8u) * 16u + ((l / 8u) & 1u) * 128u + (l / 8u) * 2048u; }},
+            {"16 groups of 4 lanes (64 B), all on banks 0-15", [](uint32_t l) { return (l % 4u) * 16u + (l / 4u) * 1024u; }},
+            {"16 groups of 4 lanes, group g on bank group g mod 4", [](uint32_t l) { return (l % 4u) * 16u + ((l / 4u) & 3u) * 64u + (l / 4u) * 1024u; }},
+            {"16 groups of 4 lanes, bank groups 0,0,1,1,2,2,3,3 repeated", [](uint32_t l) { return (l % 4u) * 16u + (((l / 4u) >> 1) & 3u) * 64u + (l / 4u) * 1024u; }},
+            {"16 groups of 4 lanes, bank groups 0,1,2,3,3,2,1,0 ...", [](uint32_t l) { const uint32_t g = l / 4u; return (l % 4u) * 16u + (((g & 4u) ? 3u - (g & 3u) : (g & 3u))) * 64u + g * 1024u; }},
+            {"tile 4x7 pixels in a 9-pixel-wide window, row-major slots", [](uint32_t l) { const uint32_t p = l / 4u; return (l % 4u) * 16u + ((p / 7u) * 9u + p % 7u) * 64u; }},
+        };
+        for (auto &pt : pats) {
+            for (int i = 0; i < 64; ++i) offs[i] = pt.addr((uint32_t)i);
+            CK(hipMemcpy(dOffs, offs.data(), 256, hipMemcpyHostToDevice));
+            run<19>(pt.what, cus, 16, 8.0 * 64 * 16, "bytes (ds_read_b128)", dOut, dCyc, dOffs, dEnts);
+        }
+        // the windowed convolution's reads: 4 lanes per output pixel (16 batch entries), 16 pixels per wave; tiles of
+        // the ResNet-18-shaped layers, pixel slots in row-major order and in the order window_pixel_order deals them
+        struct { const char *what; uint32_t TH, TW, IW, sth, stw; } tiles[] = {
+            {"tile 4x8, window row 10 pixels (56x56 3x3 layers)", 4, 8, 10, 1, 1},
+            {"tile 4x7, window row 9 (28x28 3x3 layers)", 4, 7, 9, 1, 1},
+            {"tile 2x7, window row 9 (14x14 and 7x7 3x3 layers)", 2, 7, 9, 1, 1},
+            {"tile 4x7, stride 2, window row 15 (3x3 stride-2 layers)", 4, 7, 15, 2, 2},
+            {"tile 4x8, stride 2, window row 21 (7x7 stride-2 stem)", 4, 8, 21, 2, 2},
+        };
+        for (auto &t : tiles)
+            for (int permuted = 0; permuted < 2; ++permuted)
+                for (uint32_t wave = 0; wave * 16u < t.TH * t.TW; ++wave) {
+                    WinArgs a{};
+                    a.TH = t.TH; a.TW = t.TW; a.IW = t.IW; a.sth = t.sth; a.stw = t.stw;
+                    window_pixel_order(a, 4);
+                    for (uint32_t l = 0; l < 64; ++l) {
+                        const uint32_t slot = wave * 16u + l / 4u;
+                        uint32_t px = slot < t.TH * t.TW ? slot : 0u;
+                        if (permuted) px = (a.order[slot >> 2] >> ((slot & 3u) * 8u)) & 0xffu;
+                        offs[l] = (l % 4u) * 16u + ((px / t.TW) * t.sth * t.IW + (px % t.TW) * t.stw) * 64u;
+                    }
+                    CK(hipMemcpy(dOffs, offs.data(), 256, hipMemcpyHostToDevice));
+                    char what[160];
+                    std::snprintf(what, sizeof what, "%s, wave %u, %s", t.what, wave, permuted ? "dealt slots" : "row-major slots");
+                    run<19>(what, cus, 16, 8.0 * 64 * 16, "bytes (ds_read_b128)", dOut, dCyc, dOffs, dEnts);
+                }
+        for (int i = 0; i < 64; ++i) offs[i] = (uint32_t)((i * 37) % 60) * 256u;
+        CK(hipMemcpy(dOffs, offs.data(), 256, hipMemcpyHostToDevice));
+    }
     for (int waves : {16, 8}) {
         run<0>("ds_read_b128, conflict-free", cus, waves, 8.0 * 64 * 16, "bytes", dOut, dCyc, dOffs, dEnts);
         run<18>("ds_write_b128, conflict-free", cus, waves, 8.0 * 64 * 16, "bytes", dOut, dCyc, dOffs, dEnts);

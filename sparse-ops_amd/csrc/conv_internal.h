@@ -83,7 +83,7 @@ inline uint32_t window_subsample(uint32_t k, uint32_t stride) { return k == 1 ? 
 // are not a multiple of 16 / lpp pixels wide (tiles 7 pixels wide: every second read takes two
 // turns).  Which slot computes which pixel is free, so the slots are dealt out such that the
 // pixels of each group of 16 / lpp slots fall on different bank groups wherever the tile's shape
-// allows it.  At most 64 pixels per tile.
+// allows it.  At most 64 pixels per tile; the table covers all 64 slots.
 inline void window_pixel_order(WinArgs &a, uint32_t lpp)
 {
     const uint32_t m = 16u / lpp, npx = a.TH * a.TW;
@@ -112,6 +112,9 @@ inline void window_pixel_order(WinArgs &a, uint32_t lpp)
             if (!any) break;
         }
     }
+    // Slots beyond the tile compute nothing but still read: they repeat an address of their own group
+    // of m slots (a read that several lanes share costs the banks one turn), or the previous group's.
+    for (uint32_t i = filled; i < 64u; ++i) slots[i] = (i % m != 0) ? slots[i - i % m] : (i >= m ? slots[i - m] : 0);
     for (uint32_t i = 0; i < 16; ++i)
         a.order[i] = (uint32_t)slots[4 * i] | ((uint32_t)slots[4 * i + 1] << 8) | ((uint32_t)slots[4 * i + 2] << 16) | ((uint32_t)slots[4 * i + 3] << 24);
 }

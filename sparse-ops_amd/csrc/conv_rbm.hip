@@ -212,7 +212,7 @@ void conv2d_rbm_kernel(const int4 *__restrict__ sets, const uint32_t *__restrict
     // this lane's output pixel and its corner inside the window
     const uint32_t pl = pgi * PPW + lane / LPP, b4 = lane % LPP;
     const bool pvalid = pl < a.TH * a.TW;
-    const uint32_t pc = pvalid ? window_slot_pixel(a, pl) : 0u;
+    const uint32_t pc = window_slot_pixel(a, pl & 63u);          // slots beyond the tile repeat a pixel of their group
     const uint32_t ty = pc / a.TW, tx = pc % a.TW;
     const bool live = computes && pvalid && th0 + ty < g.H_out && tw0 + tx < g.W_out;
     const uint32_t lanebase = ((ty * a.sth * a.IW + tx * a.stw) << SHIFT) + b4 * 16u;   // bytes

@@ -310,7 +310,8 @@ def test_resnet18_full_size_batch_independence(backend, oracle, tmp_path):
 def test_cpp_caller_of_the_reference_headers(oracle, tmp_path):
     """tests/cpp/dropin_consumer.cpp is a C++ program written against the reference's headers
     (host pointers, as its benchmark drivers call the kernels): encoder round trip, ellpack_matmul
-    and the fused-ReLU instantiation bit for bit, ellpack_matvec within 1e-5, and
+    and the fused-ReLU instantiation bit for bit, ellpack_matvec within 1e-5, the in-place activations, the four
+    conv2d_* entry points of conv_kernels.hpp on their three layouts (with and without the RBM plan), and
     SparseOnnxModel::run / resize_buffers on a Gemm+ReLU chain bit for bit against the oracle."""
     import subprocess
     exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "dropin_consumer")
@@ -328,7 +329,7 @@ def test_cpp_caller_of_the_reference_headers(oracle, tmp_path):
     r = subprocess.run([exe, path, str(tmp_path / "in.bin"), str(tmp_path / "expected.bin"), str(B)],
                        capture_output=True, text=True, timeout=100)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("ok  ") == 10 and "FAIL" not in r.stdout
+    assert r.stdout.count("ok  ") == 16 and "FAIL" not in r.stdout
 
 
 def _run_device(model, ctx, X_bm):
