@@ -190,6 +190,27 @@ __device__ __forceinline__ void rbm_steps(f32x32 &acc, const int4 *sets, uint32_
           "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67");
 }
 
+// Brings `lines` 64-byte lines from `p` on into the scalar cache: one scalar load per line, all in
+// flight together, then one wait.  The step loop's own scalar loads then hit, which shortens the wait
+// they share with the LDS reads (measured: 56x56x64 layer at batch 32 from 67 to 64 us, 7x7 stem from
+// 98 to 89 us).
+__device__ __forceinline__ void rbm_touch(const int4 *p, uint32_t lines)
+{
+    uint32_t sink;
+    asm volatile(
+        "L_rbm_touch_%=:\n\t"
+        "s_load_dword %[d], s[34:35], 0x0\n\t"
+        "s_add_u32 s34, s34, 64\n\t"
+        "s_addc_u32 s35, s35, 0\n\t"
+        "s_sub_u32 %[n], %[n], 1\n\t"
+        "s_cmp_lg_u32 %[n], 0\n\t"
+        "s_cbranch_scc1 L_rbm_touch_%=\n\t"
+        "s_waitcnt lgkmcnt(0)\n\t"
+        : [d] "=&s"(sink), "+{s[34:35]}"(p), [n] "+s"(lines)
+        :
+        : "scc");
+}
+
 template <int LPP, int ACT>
 __global__ __launch_bounds__(kWinThreads)
 void conv2d_rbm_kernel(const int4 *__restrict__ sets, const uint32_t *__restrict__ gbase,
@@ -271,6 +292,10 @@ void conv2d_rbm_kernel(const int4 *__restrict__ sets, const uint32_t *__restrict
 
     const int4 *__restrict__ sp = sets + (size_t)gbase[gi] * (kRbmSetBytes / 16);
     const uint32_t *__restrict__ cp = counts + (size_t)gi * a.nch;
+    {
+        const uint32_t n0 = computes ? __builtin_amdgcn_readfirstlane(cp[0]) : 0u;
+        if (n0) rbm_touch(sp, n0 + 1u);              // a set is one line; the loop requests one set past the last
+    }
     __syncthreads();
 
     for (uint32_t t = 0; t < a.nch; ++t) {
@@ -281,6 +306,10 @@ void conv2d_rbm_kernel(const int4 *__restrict__ sets, const uint32_t *__restrict
         if (n != 0u) {
             rbm_steps<(int)SHIFT>(acc, sp, n, lanebase + cur_buf * buf_bytes);
             sp += (size_t)n * (kRbmSetBytes / 16);
+        }
+        if (more) {                                  // the next chunk's sets, while the slower waves finish this one
+            const uint32_t nn = computes ? __builtin_amdgcn_readfirstlane(cp[t + 1]) : 0u;
+            if (nn) rbm_touch(sp, nn + 1u);
         }
         if (a.nbuf == 2) {
             if (more) store_window(cur_buf ^ 1u);
@@ -343,13 +372,15 @@ void rbm_launch_act(so_ctx *ctx, const so_conv_plan *plan, const WinArgs &a, dim
 }
 
 // A wave of this kernel owns a whole block of channels, so a launch has an eighth of the waves the
-// per-row kernel can spread over the chip: it pays once the grid covers about three quarters of the
-// compute units (measured on ResNet-18-shaped layers: 56x56x64 at batch 32, 196 workgroups, 66 against
-// 69 us; 28x28x128 at batch 128, 448 workgroups, 227 against 250 us) and loses below (28x28x128 at
-// batch 32, 112 workgroups: 114 against 69 us).
-bool rbm_pays(const so_ctx *ctx, uint64_t workgroups)
+// per-row kernel can spread over the chip: it needs a grid that covers about three quarters of the
+// compute units (28x28x128 at batch 32, 112 workgroups: 113 against 66 us).  With such a grid it is
+// level with the per-row kernel on stride-1 layers (ResNet-18 shapes, 3x3: 56x56x64 at batch 32 64.4
+// against 62.9 us, at batch 128 256 against 258; 28x28x128 at batch 128 224 against 219) and ahead
+// on strided ones (7x7 stride-2 stem 87 against 99 us at batch 32, 299 against 339 at batch 128;
+// 3x3 stride-2 56->28 at batch 64 71 against 80; 1x1 stride-2 18 against 19): it runs there.
+bool rbm_pays(const so_ctx *ctx, const so_conv_geom &g, uint64_t workgroups)
 {
-    return 4ull * workgroups >= 3ull * (uint64_t)ctx->compute_units;
+    return 4ull * workgroups >= 3ull * (uint64_t)ctx->compute_units && (g.stride_h > 1 || g.stride_w > 1);
 }
 
 } // namespace
@@ -514,7 +545,7 @@ so_status so_conv_rbm_launch(so_ctx *ctx, const so_conv_plan *plan, const float 
     if (a.win_f4 > (uint32_t)kRbmMaxPerThread * kWinThreads) return SO_OK;      // this kernel copies at most that many elements per thread
     const dim3 grid(w.tiles_x * w.tiles_y, so_ceil_div(a.groups, a.cg), B / (4 * LPP));
     if (grid.y > 65535u || grid.z > 65535u) return SO_OK;
-    if (!forced && !rbm_pays(ctx, (uint64_t)grid.x * grid.y * grid.z)) return SO_OK;
+    if (!forced && !rbm_pays(ctx, plan->g, (uint64_t)grid.x * grid.y * grid.z)) return SO_OK;
     switch (LPP) {
     case 4:  rbm_launch_act<4>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
     case 2:  rbm_launch_act<2>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
