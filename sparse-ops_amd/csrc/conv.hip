@@ -385,6 +385,44 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
         for (int c = 0; c < CPW; ++c) nq[c] = computes ? qp[t * CPW + c] : 0u;
 #pragma unroll
         for (int c = 0; c < CPW; ++c) {
+            if constexpr (LANE_ENT && CPW <= 2) {
+                // Pipelined: a quad's LDS reads overlap the previous quad's multiply-adds all through
+                // the run (so_dpp::group16).  Measured on ResNet-18 shapes at batch 32: 14x14x256
+                // (2 channels per wave) 63.5 -> 58.4 us, 7x7x512 (1 per wave) 69.1 -> 66.1 us; with 4
+                // channels per wave the four copies of these bodies made 28x28x128 11 % slower.
+                const uint32_t n = nq[c];
+                const char *xb = lds_bytes + base;
+                float4 xA[4], xB[4];
+                if (n >= 4u) {
+                    ep += 16;
+                    int2 enxt = ep[0];                                    // the stream ends with 16 padding entries
+                    so_dpp::group16<false>(xb, __int_as_float(ecur.x), (uint32_t)ecur.y << SHIFT, 0.0f, xA, xB, acc[c]);
+                    float ewp = __int_as_float(ecur.x);
+                    ecur = enxt;
+                    uint32_t q = 4u;
+                    for (; q + 4u <= n; q += 4u) {
+                        ep += 16;
+                        enxt = ep[0];
+                        so_dpp::group16<true>(xb, __int_as_float(ecur.x), (uint32_t)ecur.y << SHIFT, ewp, xA, xB, acc[c]);
+                        ewp = __int_as_float(ecur.x);
+                        ecur = enxt;
+                    }
+                    if (q < n) {
+                        ep += 4u * (n - q);
+                        enxt = ep[0];
+                        so_dpp::group_tail<true>(n - q, xb, __int_as_float(ecur.x), (uint32_t)ecur.y << SHIFT, ewp, xA, xB, acc[c]);
+                        ecur = enxt;
+                    } else {
+                        so_dpp::group_drain(ewp, xB, acc[c]);
+                    }
+                } else if (n != 0u) {
+                    ep += 4u * n;
+                    const int2 enxt = ep[0];
+                    so_dpp::group_tail<false>(n, xb, __int_as_float(ecur.x), (uint32_t)ecur.y << SHIFT, 0.0f, xA, xB, acc[c]);
+                    ecur = enxt;
+                }
+                continue;
+            }
             if constexpr (LANE_ENT) {
                 for (uint32_t q = 0; q < nq[c]; q += 4u) {
                     const uint32_t steps = 4u * min(4u, nq[c] - q);      // this group: 4, 8, 12 or 16 entries

@@ -77,4 +77,74 @@ __device__ __forceinline__ void tiled_chunk(const char *base, float ew, uint32_t
     }
 }
 
+// ---- the same steps, software-pipelined ------------------------------------------------
+//
+// Four steps (a quad) at a time: the quad's four LDS reads go out, and while they are in flight the
+// previous quad's sixteen multiply-adds run on operands that have already arrived.  LDS returns data
+// in order, so the wait in front of a quad's multiply-adds leaves the next quad's four reads in
+// flight.  Two operand buffers, A and B; between groups of sixteen steps the quad still owed its
+// multiply-adds sits in B.  The scheduling fences keep the compiler from moving a quad's
+// multiply-adds back in front of the reads that are meant to overlap them.  One straight-line body
+// per group length: a branch around reads would make the compiler's wait counts assume the path with
+// the fewest reads in flight, which turns every later wait into a full one.
+template <int N0>
+__device__ __forceinline__ void quad_read(const char *base, uint32_t eoff, float4 (&x)[4])
+{
+    StepRange<N0, N0 + 4>::read(base, eoff, x);
+    __builtin_amdgcn_sched_barrier(0);
+}
+template <int N0>
+__device__ __forceinline__ void quad_fma(float ew, const float4 (&x)[4], float (&acc)[4])
+{
+    StepRange<N0, N0 + 4>::fma(ew, x, acc);
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// A full group of sixteen steps.  OWED: quad 3 of the previous group (pairs in ewp, operands in xB)
+// still has its multiply-adds to do.  Leaves this group's quad 3 owed, operands in xB.
+template <bool OWED>
+__device__ __forceinline__ void group16(const char *base, float ew, uint32_t eoff, float ewp, float4 (&xA)[4], float4 (&xB)[4],
+                                        float (&acc)[4])
+{
+    asm volatile("s_nop 4" : "+v"(ew), "+v"(eoff));       // DPP operands: not within two cycles of a vector write
+    quad_read<0>(base, eoff, xA);
+    if constexpr (OWED) quad_fma<12>(ewp, xB, acc);
+    quad_read<4>(base, eoff, xB);
+    quad_fma<0>(ew, xA, acc);
+    quad_read<8>(base, eoff, xA);
+    quad_fma<4>(ew, xB, acc);
+    quad_read<12>(base, eoff, xB);
+    quad_fma<8>(ew, xA, acc);
+}
+
+// The last group of a run: `quads` (1..3) quads, then nothing is owed any more.
+template <bool OWED>
+__device__ __forceinline__ void group_tail(uint32_t quads, const char *base, float ew, uint32_t eoff, float ewp, float4 (&xA)[4],
+                                           float4 (&xB)[4], float (&acc)[4])
+{
+    asm volatile("s_nop 4" : "+v"(ew), "+v"(eoff));
+    quad_read<0>(base, eoff, xA);
+    if constexpr (OWED) quad_fma<12>(ewp, xB, acc);
+    if (quads == 1u) {
+        quad_fma<0>(ew, xA, acc);
+    } else {
+        quad_read<4>(base, eoff, xB);
+        quad_fma<0>(ew, xA, acc);
+        if (quads == 2u) {
+            quad_fma<4>(ew, xB, acc);
+        } else {
+            quad_read<8>(base, eoff, xA);
+            quad_fma<4>(ew, xB, acc);
+            quad_fma<8>(ew, xA, acc);
+        }
+    }
+}
+
+// The multiply-adds still owed after a run's last full group.
+__device__ __forceinline__ void group_drain(float ewp, const float4 (&xB)[4], float (&acc)[4])
+{
+    asm volatile("s_nop 1" : "+v"(ewp));
+    quad_fma<12>(ewp, xB, acc);
+}
+
 } // namespace so_dpp
