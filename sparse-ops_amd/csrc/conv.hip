@@ -260,6 +260,23 @@ __device__ __forceinline__ void touch_stream(const int4 *p, uint32_t quads)
         : "scc");
 }
 
+// The four waves that share a SIMD are served oldest first: left alone, the first of them finishes a
+// chunk's steps in half the time of the last (measured with the shader clock on the 56x56x64 layer:
+// 14.1 k, 17.4 k, 22.1 k, 28.7 k clocks by age), and everybody then waits for the last one at the
+// chunk's barrier with the SIMD mostly idle.  Each wave therefore keeps taking a new priority, the
+// four of a SIMD four different ones at the same point of their work (wave / 4 is the wave's age rank
+// on its SIMD).  Measured at batch 32: 56x56x64 layer 63.1 -> 58.5 us, 28x28x128 67.3 -> 65.1,
+// 14x14x256 60.2 -> 58.4; inside the 8-channel form's quad loop the extra branch costs what it gains.
+__device__ __forceinline__ void rotate_priority(uint32_t turn)
+{
+    switch (turn & 3u) {
+    case 0: __builtin_amdgcn_s_setprio(0); break;
+    case 1: __builtin_amdgcn_s_setprio(1); break;
+    case 2: __builtin_amdgcn_s_setprio(2); break;
+    default: __builtin_amdgcn_s_setprio(3); break;
+    }
+}
+
 template <int CPW, int LPP, int ACT>
 __global__ __launch_bounds__(kWinThreads)
 void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__restrict__ gbase,
@@ -357,6 +374,8 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
     // ResNet-18-shaped stack: 5-11 % faster per layer with 1 or 2 channels per wave, equal with 4,
     // 9 % slower with 8 (batch 32); 8-13 % faster over the whole stack at batches 1 to 16.
     constexpr bool LANE_ENT = CPW < 8;
+    // priorities rotate on the full batch tile only: on the smaller ones (batches below 16) it measured 5 % slower
+    constexpr bool ROTATE = LPP == 4;
     const int2 *__restrict__ ep = reinterpret_cast<const int2 *>(sp0) + (lane & 15u);
     int2 ecur = make_int2(0, 0);
     uint32_t qtouch = 0;                                             // quads of the chunk about to start
@@ -385,6 +404,8 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
         for (int c = 0; c < CPW; ++c) nq[c] = computes ? qp[t * CPW + c] : 0u;
 #pragma unroll
         for (int c = 0; c < CPW; ++c) {
+            const uint32_t turn = (wave >> 2) + (uint32_t)c + t;      // a new priority per run; per group of 16 entries where the entries sit in lanes
+            if constexpr (ROTATE) rotate_priority(turn);
             if constexpr (LANE_ENT && CPW <= 2) {
                 // Pipelined: a quad's LDS reads overlap the previous quad's multiply-adds all through
                 // the run (so_dpp::group16).  Measured on ResNet-18 shapes at batch 32: 14x14x256
@@ -401,6 +422,7 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
                     ecur = enxt;
                     uint32_t q = 4u;
                     for (; q + 4u <= n; q += 4u) {
+                        if constexpr (ROTATE) rotate_priority(turn + (q >> 2));
                         ep += 16;
                         enxt = ep[0];
                         so_dpp::group16<true>(xb, __int_as_float(ecur.x), (uint32_t)ecur.y << SHIFT, ewp, xA, xB, acc[c]);
@@ -425,6 +447,7 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
             }
             if constexpr (LANE_ENT) {
                 for (uint32_t q = 0; q < nq[c]; q += 4u) {
+                    if (ROTATE && q) rotate_priority(turn + (q >> 2));
                     const uint32_t steps = 4u * min(4u, nq[c] - q);      // this group: 4, 8, 12 or 16 entries
                     ep += steps;
                     const int2 enxt = ep[0];                              // the stream ends with 16 padding entries
