@@ -3,6 +3,7 @@
 // measured 1 % faster for this kernel and 10 % slower for the row kernel's few-wave variant.
 #include "so_internal.h"
 #include "dpp_steps.h"
+#include "lds_sync.h"
 
 namespace {
 
@@ -109,6 +110,12 @@ void ellpack_matmul_tiled_kernel(const so_tile_entry *__restrict__ entries, cons
     if (!quad_ok) cur.steps = 0;
     eload(cur, ew, eo);
     if (tid < 16) *reinterpret_cast<float4 *>(lds + so_tiled::kZeroRowOff + tid * 16) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    // Progress counters instead of a barrier per tile (lds_sync.h): [0], [1] tiles stored into buffer
+    // 0 / 1 (x 16 waves), [2], [3] tiles read out of them.  Measured on the 4096 x 4096 @ 90 % x 256
+    // launch: 39.7 -> 37.8 us (storing after the second chunk instead of the first: 43.4).
+    static_assert(so_tiled::kSyncOff + so_lds::kSyncBytes <= so_tiled::kLdsBytes, "room for the counters");
+    const uint32_t sync_base = so_lds::lds_address(lds + so_tiled::kSyncOff);
+    if (tid < 4) reinterpret_cast<uint32_t *>(lds + so_tiled::kSyncOff)[tid] = tid == 0 ? 16u : 0u;
     gload(0);
     lstore(0);
     __syncthreads();
@@ -123,15 +130,23 @@ void ellpack_matmul_tiled_kernel(const so_tile_entry *__restrict__ entries, cons
             gload(t + 1);
         }
         const char *base = lds + (t & 1u) * TILE + lane_off;
+        const bool more = t + 1 < ntiles;
 #pragma unroll
-        for (int c = 0; c < kMaxChunks; ++c)
+        for (int c = 0; c < kMaxChunks; ++c) {
+            if (c == 1 && more) {
+                // the wave's part of the next tile, once every wave has finished the tile before this one
+                so_lds::wait(sync_base + 8u + ((t + 1u) & 1u) * 4u, 16u * ((t + 1u) / 2u));
+                lstore((t + 1) & 1u);
+                so_lds::signal(sync_base + ((t + 1u) & 1u) * 4u, lane);
+            }
             if (cur.steps > 16u * c) so_dpp::tiled_chunk(base, ew[c], eo[c], cur.steps - 16u * c, acc);
+        }
         for (uint32_t c = kMaxChunks; c * 16u < cur.steps; ++c) {
             const so_tile_entry e = lane_ent[(size_t)(cur.chunk0 + c) * 64];
             so_dpp::tiled_chunk(base, e.w, e.off, cur.steps - 16u * c, acc);
         }
-        if (t + 1 < ntiles) lstore((t + 1) & 1u);
-        __syncthreads();
+        so_lds::signal(sync_base + 8u + (t & 1u) * 4u, lane);                                     // done reading this tile's buffer
+        if (more) so_lds::wait(sync_base + ((t + 1u) & 1u) * 4u, 16u * ((t + 1u) / 2u + 1u));     // the next tile is complete
         cur = nxt;
 #pragma unroll
         for (int c = 0; c < kMaxChunks; ++c) { ew[c] = nw[c]; eo[c] = no[c]; }

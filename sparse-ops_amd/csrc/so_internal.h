@@ -59,7 +59,8 @@ struct so_tiled {
     static constexpr uint32_t kSlabCols = 64;    // dense columns per workgroup
     static constexpr uint32_t kTileBytes = kTileRows * kSlabCols * 4;
     static constexpr uint32_t kZeroRowOff = 2 * kTileBytes;      // after the two tile buffers
-    static constexpr uint32_t kLdsBytes = 2 * kTileBytes + kSlabCols * 4;
+    static constexpr uint32_t kSyncOff = kZeroRowOff + kSlabCols * 4;    // the workgroup's progress counters (csrc/lds_sync.h)
+    static constexpr uint32_t kLdsBytes = kSyncOff + 64;
     uint32_t nquads = 0, ntiles = 0;
     uint64_t total_steps = 0;
     so_tile_entry *d_entries = nullptr;   // [chunks + 3][64]
