@@ -231,7 +231,7 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
 // groups and a wave accumulates CPW output channels.  The batch tile is 16 (LPP = 4): measured
 // against 32 and 8 it was the fastest on every layer of the ResNet-18-shaped stack, because the
 // smaller window lets a chunk hold twice the channels (longer runs per channel, half the barriers).  Entries are wave-uniform.  With
-// 8 channels per wave they arrive through scalar loads, four at a time and one quad ahead, so
+// 8 or 4 channels per wave they arrive through scalar loads, four at a time and one quad ahead, so
 // the weight is a scalar operand of the multiply-adds and the tap offset a scalar addend of the
 // LDS address; with fewer channels per wave (fewer, longer runs and usually fewer waves to hide
 // a scalar load behind) they are held one per lane and handed round by DPP (dpp_steps.h), 16
@@ -372,11 +372,12 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
     i32x4 cur0 = {0, 0, 0, 0}, cur1 = cur0;
     // LANE_ENT: the entries sit in lanes instead (lane l of every 16-lane row holds entry l of the
     // next 16), fetched with vector loads one group ahead and broadcast by DPP: vector loads have
-    // their own counter, so waiting for LDS data never waits for entries, which is what bounds the
-    // scalar path when there are too few waves to hide the scalar loads' latency.  Measured on a
-    // ResNet-18-shaped stack: 5-11 % faster per layer with 1 or 2 channels per wave, equal with 4,
-    // 9 % slower with 8 (batch 32); 8-13 % faster over the whole stack at batches 1 to 16.
-    constexpr bool LANE_ENT = CPW < 8;
+    // their own counter, so waiting for LDS data never waits for entries.  A DPP multiply-add keeps
+    // the vector unit busy a third longer than one with a scalar weight, though, so the scalar form
+    // wins wherever a wave has enough runs per chunk to amortise its scalar loads: measured on the
+    // ResNet-18-shaped layers at batch 32, scalar against lanes: 8 channels per wave 55 against 60 us,
+    // 4 channels 56.1 against 63.2, 2 channels 58.8 against 56.6; small batches use 1-2 channels.
+    constexpr bool LANE_ENT = CPW < 4;
     // priorities rotate on the full batch tile only: on the smaller ones (batches below 16) it measured 5 % slower
     constexpr bool ROTATE = LPP == 4;
     // progress counters instead of a barrier per chunk: the same (batch 8: 0.466 -> 0.474 ms, batch 1: 0.365 -> 0.374 with them)
