@@ -29,7 +29,7 @@ COPY_KIB = 262144.0      # bench.py --calibrate-copy: 256 MiB read, 256 MiB writ
 # bench.py reports a kernel's traffic only while the hash still matches.
 KERNEL_SOURCES = {
     "ellpack_matmul_tiled_kernel": ["sparse-ops_amd/csrc/matmul_tiled.hip", "sparse-ops_amd/csrc/dpp_steps.h",
-                                    "sparse-ops_amd/csrc/so_internal.h"],
+                                    "sparse-ops_amd/csrc/lds_sync.h", "sparse-ops_amd/csrc/so_internal.h"],
     "ellpack_matmul_kernel": ["sparse-ops_amd/csrc/matmul.hip", "sparse-ops_amd/csrc/so_internal.h"],
     "matvec_rows_kernel": ["sparse-ops_amd/csrc/matvec.hip"],
     "matvec_binned_kernel": ["sparse-ops_amd/csrc/matvec.hip"],
