@@ -105,6 +105,39 @@ def test_conv_lds_window_kernel(ctx, oracle, Cin, Cout, H, Wi, B, k, s, p, d, sp
     assert rel_err(gpu_conv(ctx, E, g, X, B, b, "tanh", window=True), oracle.conv2d_pf(as_oracle(E), og, X, B, b, "tanh")) <= 1e-6
 
 
+@pytest.mark.parametrize("Cin,Cout,H,B,sp", [(64, 64, 28, 32, .8), (256, 96, 7, 16, .8), (96, 40, 14, 48, .7)])
+def test_conv_lds_window_kernel_many_launches(ctx, oracle, Cin, Cout, H, B, sp):
+    """Several chunks per workgroup on the 16-entry batch tile: the waves synchronise through
+    progress counters in LDS instead of barriers.  Every one of many back-to-back launches gives
+    the oracle's bits (a race between a window's stores and its reads would show up as a launch
+    that differs)."""
+    from oracle import conv_geom as ocg
+    rng = np.random.default_rng(Cin + Cout + H)
+    Wc = sparse_matrix(rng, Cout, Cin * 9, sp)
+    X = rng.standard_normal((Cin, H, H, B)).astype(np.float32)
+    b = rng.standard_normal(Cout).astype(np.float32)
+    E = datagen.encode_dense(Wc)
+    g, og = hipabi.conv_geom(Cin, Cout, 3, 3, H, H, (1, 1), (1, 1), (1, 1)), ocg(Cin, Cout, 3, 3, H, H, (1, 1), (1, 1), (1, 1))
+    Yo = oracle.conv2d_pf(as_oracle(E), og, X, B, b, "relu")
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r)
+    plan = ctx.conv_plan(dE, g)
+    ctx.conv_plan_tune(plan, B)
+    win = ctx.conv_plan_window(plan)
+    assert win is not None and win["chunks"] >= 2
+    dX, dB = ctx.array(X), ctx.array(b)
+    outs = [ctx.empty((Cout, g.H_out, g.W_out, B)) for _ in range(4)]
+    with ctx.tuning(SPARSEOPS_CONV_WINDOW="1"):
+        for rep in range(25):
+            for dY in outs:                                  # four launches in flight behind one another
+                ctx.conv2d(plan, dX, B, dB, dY, "relu")
+            for dY in outs:
+                assert np.array_equal(dY.download(), Yo), "launch %d differs" % rep
+    ctx.conv_plan_free(plan)
+    dE.free()
+    for a in [dX, dB] + outs:
+        a.free()
+
+
 @pytest.mark.parametrize("B,window", [(3, False), (4, False), (32, False), (32, True), (16, True), (8, True), (4, True)])
 def test_conv_with_fused_residual_add(ctx, oracle, B, window):
     """so_conv2d_add == conv, then the reference's Add, then the activation: same bits as

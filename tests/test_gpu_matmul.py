@@ -158,6 +158,31 @@ def test_matmul_lds_tiled_reference_vectors_and_config3(ctx, oracle, golden):
     assert np.isfinite(Yi[rows_without_col0]).all() and np.array_equal(Yi[rows_without_col0], Y[rows_without_col0])
 
 
+@pytest.mark.parametrize("m,n,C,sp", [(1024, 2048, 256, .9), (200, 1300, 64, .7), (64, 5000, 128, .95)])
+def test_matmul_lds_tiled_many_launches(ctx, oracle, m, n, C, sp):
+    """Several K-tiles per workgroup: the waves synchronise through progress counters in LDS
+    instead of a barrier per tile.  Every one of many back-to-back launches gives the oracle's
+    bits (a race between a tile's stores and its reads would show up as a launch that differs)."""
+    rng = np.random.default_rng(m + n + C)
+    W = sparse_matrix(rng, m, n, sp)
+    X = rng.standard_normal((n, C)).astype(np.float32)
+    b = rng.standard_normal(m).astype(np.float32)
+    E = datagen.encode_dense(W)
+    Yo = oracle.matmul(as_oracle(E), X, b)
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, TILED)
+    dX, dB = ctx.array(X), ctx.array(b)
+    outs = [ctx.empty((m, C)) for _ in range(4)]
+    with ctx.tuning(SPARSEOPS_MATMUL_TILED="1"):
+        for rep in range(25):
+            for dY in outs:                                  # four launches in flight behind one another
+                ctx.matmul(dE, dX, C, dB, dY, "none")
+            for dY in outs:
+                assert np.array_equal(dY.download(), Yo), "launch %d differs" % rep
+    dE.free()
+    for a in [dX, dB] + outs:
+        a.free()
+
+
 def test_matmul_lds_tiled_keeps_negative_zero(ctx, oracle):
     """Rows that share a wave with longer rows run padding steps; those must leave a
     -0.0 accumulator (bias -0.0, no contribution yet) as it is, sign bit included."""
