@@ -11,19 +11,20 @@ namespace {
 // LDS-staged variant (SO_LAYOUT_TILED).
 //
 // The row kernel above moves every X operand through the vector L1, which
-// sustains about 50 bytes/clk per CU; LDS sustains three times that for 16-byte
-// reads.  Here a workgroup of 16 waves owns 64 rows and one slab of 64 dense
+// sustains about 50 bytes/clk per CU; LDS sustains five times that for 16-byte
+// reads (255 bytes/clk per CU measured).  Here a workgroup of 16 waves owns 64 rows and one slab of 64 dense
 // columns, and streams the slab X[:, c0..c0+64) through LDS in tiles of 256 rows
 // (64 KB, double-buffered: the next tile is fetched into registers while the
-// current one is consumed).  A wave works on a quad of four rows, 16 lanes per
+// current one is consumed; progress counters in LDS, not barriers, tell a wave when
+// a buffer may be read or overwritten).  A wave works on a quad of four rows, 16 lanes per
 // row, four columns per lane, so one ds_read_b128 per lane serves four FMAs.  The
 // (weight, LDS offset) pairs of a quad's rows for the current tile sit in lanes
 // (chunk of 16 steps per row, fetched one tile ahead and before the X prefetch,
 // so waiting for them never waits for X) and are broadcast inside each 16-lane
 // row with DPP row_newbcast.  Each row still receives its nonzeros in ascending
 // slot order starting from the bias: results are bit-identical to the row kernel.
-// A step that a row of the quad does not have is the pair (0, zero row):
-// fma(0, 0, acc) leaves acc unchanged.
+// A step that a row of the quad does not have is the pair (-0, zero row):
+// fma(-0, 0, acc) leaves acc unchanged, a -0 accumulator included.
 // ---------------------------------------------------------------------------
 
 constexpr int kTiledWaves = so_tiled::kWavesPerGroup;
