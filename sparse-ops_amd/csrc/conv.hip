@@ -817,6 +817,8 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
 
 } // namespace
 
+uint32_t so_conv_wait_timeouts() { return so_lds::take_wait_timeouts(); }
+
 extern "C" so_status so_conv_plan_create(so_ctx *ctx, const so_ellpack *E, const so_conv_geom *g,
                                          so_conv_plan **out)
 {

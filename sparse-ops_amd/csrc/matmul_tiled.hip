@@ -180,6 +180,8 @@ so_status launch_tiled(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32
 
 } // namespace
 
+uint32_t so_matmul_wait_timeouts() { return so_lds::take_wait_timeouts(); }
+
 so_status so_matmul_tiled_launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
                                  const float *dBias, float *dY, int act)
 {

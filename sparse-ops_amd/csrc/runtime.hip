@@ -217,6 +217,12 @@ extern "C" so_status so_sync(so_ctx *ctx)
     SO_REQUIRE(ctx != nullptr, "so_sync: ctx is null");
     SO_REQUIRE(!ctx->capturing, "so_sync: not allowed while a graph is being recorded");
     SO_HIP(hipStreamSynchronize(ctx->stream));
+    // a kernel whose waves gave up waiting for one another has produced garbage: say so
+    const uint32_t gave_up = so_conv_wait_timeouts() + so_matmul_wait_timeouts();
+    if (gave_up) {
+        so_set_error("so_sync: %u waits on LDS progress counters timed out in earlier launches; their results are invalid", gave_up);
+        return SO_ERR_HIP;
+    }
     return SO_OK;
 }
 

@@ -106,6 +106,10 @@ void so_set_error(const char *fmt, ...);
 so_status so_matmul_tiled_launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
                                  const float *dBias, float *dY, int act);
 
+// Waits on LDS progress counters (csrc/lds_sync.h) that gave up since the last call; so_sync() reports them.
+uint32_t so_conv_wait_timeouts();
+uint32_t so_matmul_wait_timeouts();
+
 // Kernels that ask for more than 48 KB of dynamic LDS must be told so once per device: this does
 // it the first time `kernel` is seen on the context's device (hipSuccess when already done).
 hipError_t so_allow_big_lds(so_ctx *ctx, const void *kernel);

@@ -132,6 +132,7 @@ def test_conv_lds_window_kernel_many_launches(ctx, oracle, Cin, Cout, H, B, sp):
                 ctx.conv2d(plan, dX, B, dB, dY, "relu")
             for dY in outs:
                 assert np.array_equal(dY.download(), Yo), "launch %d differs" % rep
+    ctx.sync()                                               # fails if a wave gave up waiting on the progress counters
     ctx.conv_plan_free(plan)
     dE.free()
     for a in [dX, dB] + outs:

@@ -178,6 +178,7 @@ def test_matmul_lds_tiled_many_launches(ctx, oracle, m, n, C, sp):
                 ctx.matmul(dE, dX, C, dB, dY, "none")
             for dY in outs:
                 assert np.array_equal(dY.download(), Yo), "launch %d differs" % rep
+    ctx.sync()                                               # fails if a wave gave up waiting on the progress counters
     dE.free()
     for a in [dX, dB] + outs:
         a.free()
