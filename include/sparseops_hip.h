@@ -106,6 +106,9 @@ so_status so_h2d(so_ctx *ctx, void *dst, const void *src, size_t bytes); /* wait
 so_status so_d2h(so_ctx *ctx, void *dst, const void *src, size_t bytes); /* waits */
 so_status so_d2d(so_ctx *ctx, void *dst, const void *src, size_t bytes);
 so_status so_fill_zero(so_ctx *ctx, void *dptr, size_t bytes); /* fill kernel, graph-safe */
+/* Waits for the context's stream.  SO_ERR_HIP if a wave of an earlier launch gave up waiting for
+ * its workgroup (the LDS-staged kernels synchronise through counters with a bounded wait instead of
+ * hanging): the results of those launches are invalid. */
 so_status so_sync(so_ctx *ctx);
 
 /* HIP-event stopwatch on the context's stream: begin records an event, end
