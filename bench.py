@@ -440,8 +440,8 @@ def main():
                      "t_lds_operands_us": round(flops / (LDS_OPERAND_PEAK_TF * 1e12) * 1e6, 2),
                      "t_bound_over_t": round(max(nbytes / (HBM_PEAK_GBS * 1e9), flops / (LDS_OPERAND_PEAK_TF * 1e12)) / (ev_ms * 1e-3), 4),
                      "binding_bound": "not HBM (t_hbm 2.7 us): LDS operand reads (10.9 us at 256 B/clk/CU) and LDS tile writes (5.6 us at the "
-                                      "measured 78 B/clk/CU), multiply-adds in DPP form at half the plain rate (15 us with padding), and the "
-                                      "barrier between the 16 tile phases"},
+                                      "measured 78 B/clk/CU), multiply-adds in DPP form at half the plain rate (19 us with padding and address adds), and "
+                                      "the waves of a workgroup waiting for one another between the 16 tile phases (a quarter of a phase)"},
     }
     if args.calibrate_copy:
         # A plain copy of known size (act_kernel<NONE>: reads N floats, writes N floats)
