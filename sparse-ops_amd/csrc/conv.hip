@@ -244,20 +244,30 @@ void conv2d_implicit_kernel(const float *__restrict__ Wd, const int2 *__restrict
 // scalar loads share one counter and scalar loads return out of order, so every wait for LDS data
 // in the step loop also waits for the scalar load in flight; touched ahead, once per chunk, those
 // loads hit (measured: 56x56x64 layer at batch 32 from 67 to 63 us).
-__device__ __forceinline__ void touch_stream(const int4 *p, uint32_t quads)
+__device__ __forceinline__ void touch_stream(const int4 *p, uint32_t quads, uint32_t part, uint32_t parts)
 {
-    uint32_t lines = (quads * 32u + 32u + 63u) / 64u, sink;      // p may sit in the middle of a line
+    // the lines of the range in groups of four (up to three lines past its end: the stream ends with
+    // padding); the waves that walk the same stream -- the pixel groups of a channel group -- take
+    // every parts-th group each
+    uint32_t groups = ((quads * 32u + 32u + 63u) / 64u + 3u) / 4u, sink;      // p may sit in the middle of a line
+    if (groups <= part) return;
+    groups = (groups - part + parts - 1u) / parts;
+    p += 16u * part;
+    const uint32_t stride = 256u * parts;
     asm volatile(
         "L_touch_%=:\n\t"
         "s_load_dword %[d], s[34:35], 0x0\n\t"
-        "s_add_u32 s34, s34, 64\n\t"
+        "s_load_dword %[d], s[34:35], 0x40\n\t"
+        "s_load_dword %[d], s[34:35], 0x80\n\t"
+        "s_load_dword %[d], s[34:35], 0xc0\n\t"
+        "s_add_u32 s34, s34, %[st]\n\t"
         "s_addc_u32 s35, s35, 0\n\t"
         "s_sub_u32 %[n], %[n], 1\n\t"
         "s_cmp_lg_u32 %[n], 0\n\t"
         "s_cbranch_scc1 L_touch_%=\n\t"
         "s_waitcnt lgkmcnt(0)\n\t"
-        : [d] "=&s"(sink), "+{s[34:35]}"(p), [n] "+s"(lines)
-        :
+        : [d] "=&s"(sink), "+{s[34:35]}"(p), [n] "+s"(groups)
+        : [st] "s"(stride)
         : "scc");
 }
 
@@ -392,7 +402,7 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
 #pragma unroll
             for (int c = 0; c < CPW; ++c) qtouch += qp[c];
         }
-        touch_stream(sp0, qtouch + 1u);
+        touch_stream(sp0, qtouch + 1u, pgi, a.pg);
         cur0 = sp[0];
         cur1 = sp[1];
         sp += 2;
@@ -504,7 +514,7 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
                 uint32_t qn = 0;
 #pragma unroll
                 for (int c = 0; c < CPW; ++c) qn += qp[(t + 1) * CPW + c];
-                if (qn) touch_stream((const int4 *)(uintptr_t)sp, qn);
+                if (qn) touch_stream((const int4 *)(uintptr_t)sp, qn, pgi, a.pg);
             }
         }
         if (DRIFT && a.nbuf == 2) {
@@ -771,8 +781,9 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     const float neg_zero = -0.0f;
     uint32_t pad_bits;
     std::memcpy(&pad_bits, &neg_zero, 4);
-    // four padding quads at the end: the kernels request entries one quad, or one group of 16, ahead
-    std::vector<int2> stream((size_t)(total_quads + 4) * 4, make_int2((int32_t)pad_bits, (int32_t)(cc * w.IH * w.IW)));
+    // twelve padding quads at the end: the kernels request entries one quad, or one group of 16, ahead,
+    // and touch the stream's cache lines four at a time
+    std::vector<int2> stream((size_t)(total_quads + 12) * 4, make_int2((int32_t)pad_bits, (int32_t)(cc * w.IH * w.IW)));
     {
         size_t pos = 0;                                            // entries written so far
         std::vector<uint32_t> next(E->m, 0);                       // next unread slot of every row
