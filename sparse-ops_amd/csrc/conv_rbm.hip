@@ -194,20 +194,29 @@ __device__ __forceinline__ void rbm_steps(f32x32 &acc, const int4 *sets, uint32_
 // flight together, then one wait.  The step loop's own scalar loads then hit, which shortens the wait
 // they share with the LDS reads (measured: 56x56x64 layer at batch 32 from 67 to 64 us, 7x7 stem from
 // 98 to 89 us).
-__device__ __forceinline__ void rbm_touch(const int4 *p, uint32_t lines)
+__device__ __forceinline__ void rbm_touch(const int4 *p, uint32_t lines, uint32_t part, uint32_t parts)
 {
-    uint32_t sink;
+    // in groups of four lines (up to three past the range: the stream ends with padding sets); the
+    // waves that walk the same stream -- the pixel groups of a block -- take every parts-th group each
+    uint32_t groups = (lines + 3u) / 4u, sink;
+    if (groups <= part) return;
+    groups = (groups - part + parts - 1u) / parts;
+    p += 16u * part;
+    const uint32_t stride = 256u * parts;
     asm volatile(
         "L_rbm_touch_%=:\n\t"
         "s_load_dword %[d], s[34:35], 0x0\n\t"
-        "s_add_u32 s34, s34, 64\n\t"
+        "s_load_dword %[d], s[34:35], 0x40\n\t"
+        "s_load_dword %[d], s[34:35], 0x80\n\t"
+        "s_load_dword %[d], s[34:35], 0xc0\n\t"
+        "s_add_u32 s34, s34, %[st]\n\t"
         "s_addc_u32 s35, s35, 0\n\t"
         "s_sub_u32 %[n], %[n], 1\n\t"
         "s_cmp_lg_u32 %[n], 0\n\t"
         "s_cbranch_scc1 L_rbm_touch_%=\n\t"
         "s_waitcnt lgkmcnt(0)\n\t"
-        : [d] "=&s"(sink), "+{s[34:35]}"(p), [n] "+s"(lines)
-        :
+        : [d] "=&s"(sink), "+{s[34:35]}"(p), [n] "+s"(groups)
+        : [st] "s"(stride)
         : "scc");
 }
 
@@ -294,7 +303,7 @@ void conv2d_rbm_kernel(const int4 *__restrict__ sets, const uint32_t *__restrict
     const uint32_t *__restrict__ cp = counts + (size_t)gi * a.nch;
     {
         const uint32_t n0 = computes ? __builtin_amdgcn_readfirstlane(cp[0]) : 0u;
-        if (n0) rbm_touch(sp, n0 + 1u);              // a set is one line; the loop requests one set past the last
+        if (n0) rbm_touch(sp, n0 + 1u, pgi, a.pg);   // a set is one line; the loop requests one set past the last
     }
     __syncthreads();
 
@@ -309,7 +318,7 @@ void conv2d_rbm_kernel(const int4 *__restrict__ sets, const uint32_t *__restrict
         }
         if (more) {                                  // the next chunk's sets, while the slower waves finish this one
             const uint32_t nn = computes ? __builtin_amdgcn_readfirstlane(cp[t + 1]) : 0u;
-            if (nn) rbm_touch(sp, nn + 1u);
+            if (nn) rbm_touch(sp, nn + 1u, pgi, a.pg);
         }
         if (a.nbuf == 2) {
             if (more) store_window(cur_buf ^ 1u);
@@ -459,8 +468,8 @@ so_status so_conv_rbm_rebuild(so_ctx *ctx, so_conv_plan *plan)
         }
         if (stream.size() / kRbmSetRecords > 0x7ffffff0ull) { so_set_error("so_conv_plan_set_rbm: stream too large"); return SO_ERR_INVALID; }
     }
-    // the loop requests one set past the last one it uses
-    for (uint32_t k = 0; k < kRbmSetRecords; ++k) stream.push_back(padrec);
+    // the loop requests one set past the last one it uses, the touches reach up to three lines further
+    for (uint32_t k = 0; k < 4 * kRbmSetRecords; ++k) stream.push_back(padrec);
 
     hipError_t e = rbm_allow_lds<4>(ctx);
     if (e == hipSuccess) e = rbm_allow_lds<2>(ctx);
