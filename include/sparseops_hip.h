@@ -63,8 +63,18 @@ enum { SO_ACT_NONE = 0, SO_ACT_RELU = 1, SO_ACT_SIGMOID = 2, SO_ACT_TANH = 3 };
  *        (same values, same ascending order inside every row) for the variant
  *        of so_matmul that stages X through LDS; costs about 1.3x the ROW
  *        arrays in HBM.  so_matmul uses it whenever it is present and C is a
- *        multiple of 4; results are bit-identical to the ROW kernel. */
-enum { SO_LAYOUT_ROW = 1, SO_LAYOUT_SLOT = 2, SO_LAYOUT_BINS = 4, SO_LAYOUT_TILED = 8 };
+ *        multiple of 4; results are bit-identical to the ROW kernel.
+ * RBM  : row-block-merged, the reference's blocked-CSC idea (include/rbm_conv.hpp:8-27,
+ *        src/layers/rbm_conv.cpp:7-73) for so_matmul: rows in blocks of 128, a block's used
+ *        columns walked once, each X row segment loaded once and multiplied into every row
+ *        of the block that has a nonzero there.  The fastest so_matmul for large matrices;
+ *        so_matmul uses it whenever it is present and the launch covers most of the chip.
+ *        Sums are taken column by column, not in a row's slot order: results agree with
+ *        the reference to fp32 round-off (max |y - ref| <= 1e-5 * max |ref|), are not
+ *        bit-identical to it, and are the same bits on every launch.  Rows may be in any
+ *        order.  Costs about 1.4x the ROW arrays in HBM; with it so_matmul keeps a
+ *        workspace in the context that grows on first use of a larger output. */
+enum { SO_LAYOUT_ROW = 1, SO_LAYOUT_SLOT = 2, SO_LAYOUT_BINS = 4, SO_LAYOUT_TILED = 8, SO_LAYOUT_RBM = 16 };
 
 typedef struct so_ctx so_ctx;         /* one device + one stream + staging arena */
 typedef struct so_ellpack so_ellpack; /* device-resident ELLPACK matrix */

@@ -286,6 +286,22 @@ extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX
     // one workgroup per (4 rows, 64 columns) at most: the grid must fit 31 bits
     SO_REQUIRE(((uint64_t)E->m / 4 + 8) * ((uint64_t)C / 64 + 1) < (1ull << 31), "so_matmul: %u x %u output is too large for one launch", E->m, C);
 
+    // The row-block-merged kernel, on handles uploaded with its layout (accurate to fp32 round-off, not
+    // bit-identical to the row order: the caller asked for it by asking for the layout).  It takes one
+    // workgroup per (128 rows, 64 columns, share of the columns), so like the LDS-staged kernel it pays
+    // when that grid covers most of the chip (SPARSEOPS_MATMUL_RBM=1 forces it, =0 forbids it).
+    if (so_matmul_rbm_applies(ctx, E, C) && dX != nullptr && (((uintptr_t)dX | (uintptr_t)dY) & 3) == 0) {
+        const uint64_t groups = (uint64_t)E->rbmm.nb * so_ceil_div(C, 64) * E->rbmm.ksplit;
+        bool rbm = 4 * groups >= 3 * (uint64_t)ctx->compute_units;
+        if (ctx->tune.matmul_rbm >= 0) rbm = ctx->tune.matmul_rbm == 1;
+        if (rbm) {
+            const so_status st = so_matmul_rbm_launch(ctx, E, dX, C, dBias, dY, act);
+            if (st != SO_OK) return st;
+            SO_LAUNCH_CHECK();
+            return SO_OK;
+        }
+    }
+
     const uintptr_t align = (uintptr_t)dX | (uintptr_t)dY;
     // The LDS-staged kernel needs whole float4 column groups.  It takes one
     // workgroup per (64 rows, 64 columns), one workgroup per CU at a time, so it pays

@@ -64,6 +64,8 @@ static void read_tuning(so_tuning &t)
     t.matmul_tiled = env_int("SPARSEOPS_MATMUL_TILED", -1);
     t.matmul_vec = env_int("SPARSEOPS_MATMUL_VEC", 0);
     t.matmul_share = env_int("SPARSEOPS_MATMUL_SHARE", -1);
+    t.matmul_rbm = env_int("SPARSEOPS_MATMUL_RBM", -1);
+    t.matmul_rbm_split = env_int("SPARSEOPS_MATMUL_RBM_SPLIT", 0);
     const int lanes = env_int("SPARSEOPS_MATVEC_LANES", 0);
     t.matvec_lanes = (lanes == 8 || lanes == 16 || lanes == 32 || lanes == 64) ? lanes : 0;
     t.conv_min_cg = env_int("SPARSEOPS_CONV_MIN_CG", 0);
@@ -125,6 +127,8 @@ extern "C" so_status so_destroy(so_ctx *ctx)
     if (ctx->stream) { (void)hipStreamSynchronize(ctx->stream); (void)hipStreamDestroy(ctx->stream); }
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+    if (ctx->mm_part) (void)hipFree(ctx->mm_part);
+    if (ctx->mm_counters) (void)hipFree(ctx->mm_counters);
     delete ctx;
     return SO_OK;
 }
@@ -309,6 +313,7 @@ static void free_ellpack_arrays(so_ellpack *E)
     if (E->tiled.d_entries) (void)hipFree(E->tiled.d_entries);
     if (E->tiled.d_info) (void)hipFree(E->tiled.d_info);
     if (E->tiled.d_rows) (void)hipFree(E->tiled.d_rows);
+    so_rbmm_free(E);
 }
 
 // Device copy of a host array with 16 zeroed bytes after the last element, so a
@@ -427,7 +432,7 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
     const size_t slots = (size_t)m * r;
     SO_REQUIRE(m == 0 || nnz != nullptr, "so_ellpack_upload: nnz is null");
     SO_REQUIRE(slots == 0 || (Wd && idx), "so_ellpack_upload: Wd/idx is null");
-    SO_REQUIRE((layouts & ~(SO_LAYOUT_ROW | SO_LAYOUT_SLOT | SO_LAYOUT_BINS | SO_LAYOUT_TILED)) == 0,
+    SO_REQUIRE((layouts & ~(SO_LAYOUT_ROW | SO_LAYOUT_SLOT | SO_LAYOUT_BINS | SO_LAYOUT_TILED | SO_LAYOUT_RBM)) == 0,
                "so_ellpack_upload: unknown layout bits 0x%x", layouts);
 
     // Validate on the host before anything reaches a kernel: every stored slot must
@@ -504,6 +509,7 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
     }
 
     if (s == SO_OK && (layouts & SO_LAYOUT_TILED) && m > 0) s = build_tiled(ctx, E, Wd, idx, nnz);
+    if (s == SO_OK && (layouts & SO_LAYOUT_RBM) && m > 0) s = so_rbmm_build(ctx, E, Wd, idx, nnz);
 
     if (s != SO_OK) {
         free_ellpack_arrays(E);

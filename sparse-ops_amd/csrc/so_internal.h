@@ -14,6 +14,8 @@ struct so_tuning {
     int matmul_tiled = -1;   // SPARSEOPS_MATMUL_TILED: 1 forces the LDS-staged kernel, 0 forbids it
     int matmul_vec = 0;      // SPARSEOPS_MATMUL_VEC: 1 or 2 columns per lane at most
     int matmul_share = -1;   // SPARSEOPS_MATMUL_SHARE: 0 forbids the shared-gather kernel for few-row launches
+    int matmul_rbm = -1;     // SPARSEOPS_MATMUL_RBM: 0 forbids the row-block-merged kernel on handles that carry its layout, 1 forces it
+    int matmul_rbm_split = 0;   // SPARSEOPS_MATMUL_RBM_SPLIT: 1, 2 or 4 workgroups per tile for RBM layouts built from now on
     int matvec_lanes = 0;    // SPARSEOPS_MATVEC_LANES: 8, 16, 32 or 64 lanes per row
     int conv_min_cg = 0;     // SPARSEOPS_CONV_MIN_CG: fewest channel groups per workgroup a small grid may shrink to (16: never shrink)
     int conv_window = -1;    // SPARSEOPS_CONV_WINDOW: 1 forces the LDS-windowed kernel, 0 forbids it
@@ -31,6 +33,11 @@ struct so_ctx {
     int max_lds_bytes = 0;   // largest LDS allocation one workgroup may ask for
     bool capturing = false;
     void *static_scratch = nullptr;   // this device's address of the library's static scratch array (so_ellpack_encode_noalloc)
+    // workspace of the row-block-merged matmul (csrc/matmul_rbm.hip): partial tiles of the workgroups that share a tile, a counter per tile
+    float *mm_part = nullptr;
+    size_t mm_part_bytes = 0;
+    uint32_t *mm_counters = nullptr;
+    size_t mm_counter_bytes = 0;
     std::string name;
     so_tuning tune;
     std::vector<const void *> big_lds_kernels;   // kernels already allowed max_lds_bytes of dynamic LDS on this device
@@ -68,6 +75,21 @@ struct so_tiled {
     uint32_t *d_rows = nullptr;           // [nquads*4] row id of each quad member (0xffffffff = none)
 };
 
+// Row-block-merged copy of the matrix for so_matmul (csrc/matmul_rbm.hip): per block of 128 rows and per
+// stream (12 waves x ksplit workgroups) a run of 256-byte records, one per loop iteration, and at the same
+// index of `w` the iteration's 64 weights.
+struct so_rbmm {
+    static constexpr uint32_t kBlockRows = 128;   // rows (accumulators) per tile
+    static constexpr uint32_t kWaves = 12;        // waves per workgroup
+    static constexpr uint32_t kMaxSplit = 4;      // most workgroups per tile
+    uint32_t nb = 0, ksplit = 1;
+    uint64_t nrec = 0;                            // records (= weight blocks), tails included
+    uint64_t slots = 0, xloads = 0;               // multiply-adds a 64-column slab costs (padding included), X row segments it loads
+    uint32_t *d_hdr = nullptr;                    // per block: iterations per class (6 dwords + 2 spare), then per stream {first record, first class}
+    uint32_t *d_rec = nullptr;
+    float *d_w = nullptr;
+};
+
 struct so_ellpack {
     uint32_t m = 0, n = 0, r = 0;
     uint64_t total_nnz = 0;
@@ -81,6 +103,7 @@ struct so_ellpack {
     uint32_t *d_idxT = nullptr;
     so_bin bins[3];              // SO_LAYOUT_BINS
     so_tiled tiled;              // SO_LAYOUT_TILED
+    so_rbmm rbmm;                // SO_LAYOUT_RBM
 };
 
 // Row-block-merged re-encoding of a matrix (include/rbm_conv.hpp:8-27 of the reference), flattened:
@@ -105,6 +128,13 @@ void so_set_error(const char *fmt, ...);
 // csrc/matmul_tiled.hip: launches the LDS-staged kernel on E's TILED copy (the caller has checked that it applies).
 so_status so_matmul_tiled_launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
                                  const float *dBias, float *dY, int act);
+
+// csrc/matmul_rbm.hip: the row-block-merged layout and its kernel.
+so_status so_rbmm_build(so_ctx *ctx, so_ellpack *E, const float *Wd, const uint32_t *idx, const uint32_t *nnz);
+void so_rbmm_free(so_ellpack *E);
+bool so_matmul_rbm_applies(const so_ctx *ctx, const so_ellpack *E, uint32_t C);
+so_status so_matmul_rbm_launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
+                               const float *dBias, float *dY, int act);
 
 // Waits on LDS progress counters (csrc/lds_sync.h) that gave up since the last call; so_sync() reports them.
 uint32_t so_conv_wait_timeouts();

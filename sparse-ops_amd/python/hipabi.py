@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "libsparseops_hip.so")
 
 SO_OK, SO_ERR_NO_DEVICE, SO_ERR_INVALID, SO_ERR_OOM, SO_ERR_HIP, SO_ERR_BOUNDS = range(6)
 ACT = {"none": 0, "relu": 1, "sigmoid": 2, "tanh": 3}
-LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS, LAYOUT_TILED = 1, 2, 4, 8
+LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS, LAYOUT_TILED, LAYOUT_RBM = 1, 2, 4, 8, 16
 
 # Every symbol include/sparseops_hip.h declares.
 SYMBOLS = (
