@@ -17,11 +17,12 @@ Registers (fixed):
   s[2:7]   iterations per class, 16 bits each (classes 6 .. 16)
   s[8:11]  X as a buffer resource (base = the slab's first column, range = to the end of X)
   s[12:15] the wave's weight blocks as a buffer resource     s[16:17] the wave's records
-  s18 byte offset of the current record (= of its weight block)   s19 row pitch of X in bytes
+  s18 byte offset of the current record (= of its weight block)
   s20 iterations left in the class - 1   s21 classes left   s22 the class the wave starts with
-  s[24:27] X rows of the iteration three ahead   s[32:63], s[64:95] accumulator indices of two iterations
+  s[24:27] byte offsets of the X rows of the iteration three ahead   s[32:63], s[64:95] accumulator indices of two iterations
 A record (256 bytes) is one iteration: 32 dwords of accumulator indices (4 slots x 8 dwords x 2
-halves, each 0xC000 | accumulator: M0's index-mode bits and offset), then the 4 X rows; its 64
+halves, each 0xC000 | accumulator: M0's index-mode bits and offset), then the byte offsets of the 4 X
+rows (row * pitch, written for the launch's pitch by a small kernel whenever the pitch changes); its 64
 weights sit at the same offset of the weight array, slot-major.
 
 Per iteration t (ring position t mod 4, index buffer t mod 2): X rows and weights of iteration
@@ -46,8 +47,6 @@ LANE4, WLANE = 166, 167
 
 def vmem(slot, jbase, off):
     o = []
-    for k in range(SLOTS):
-        o.append(f"s_mul_i32 s{jbase + k}, s{jbase + k}, s19")
     for k in range(SLOTS):
         o.append(f"buffer_load_dword v{XR[slot] + k}, v{LANE4}, s[8:11], s{jbase + k} offen")
     o.append(f"buffer_load_dwordx4 v[{WR[slot]}:{WR[slot] + 3}], v{WLANE}, s[12:15], s18 offen offset:{off}")

@@ -103,11 +103,11 @@ void ellpack_matmul_rbm_kernel(const uint32_t *__restrict__ hdr, const uint32_t 
 #pragma unroll
     for (int i = 0; i < 32; ++i) { a0[i] = 0.f; a1[i] = 0.f; a2[i] = 0.f; a3[i] = 0.f; }
     uint32_t off = 0, cnt = 0, left = NCLASS;
-    const uint32_t pitch = C * 4u, lane4 = lane * 4u, wlane = (lane & 15u) * 16u;
+    const uint32_t lane4 = lane * 4u, wlane = (lane & 15u) * 16u;
     asm volatile(SO_RBMM_STEPS_ASM
                  : "+{v[4:35]}"(a0), "+{v[36:67]}"(a1), "+{v[68:99]}"(a2), "+{v[100:131]}"(a3), "+{s18}"(off), "+{s20}"(cnt), "+{s21}"(left), "+{s22}"(entry)
                  : "{s2}"(q0), "{s3}"(q1), "{s4}"(q2), "{s5}"(q3), "{s6}"(q4), "{s7}"(q5), "{s[8:11]}"(xr), "{s[12:15]}"(wr), "{s[16:17]}"(recp),
-                   "{s19}"(pitch), "{v166}"(lane4), "{v167}"(wlane)
+                   "{v166}"(lane4), "{v167}"(wlane)
                  : "memory", "scc", "m0", SO_RBMM_VCLOB, SO_RBMM_SCLOB);
 
     // The 12 partial tiles of the workgroup, added through LDS: groups of 4 rows (one 16-byte
@@ -168,6 +168,14 @@ void ellpack_matmul_rbm_kernel(const uint32_t *__restrict__ hdr, const uint32_t 
     }
 }
 
+// The records address X rows by byte offset (row * pitch): written here for the pitch of the launch at hand,
+// once per handle and pitch.
+__global__ void rbmm_offsets_kernel(uint32_t *__restrict__ rec, const uint32_t *__restrict__ xrows, uint64_t nrec, uint32_t pitch)
+{
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < nrec * 4) rec[(i >> 2) * RECDW + 32 + (i & 3)] = xrows[i] * pitch;
+}
+
 template <int ACT>
 so_status launch_rbm(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, const float *dBias, float *dY)
 {
@@ -196,7 +204,7 @@ so_status so_rbmm_build(so_ctx *ctx, so_ellpack *E, const float *Wd, const uint3
     if (ctx->tune.matmul_rbm_split == 1 || ctx->tune.matmul_rbm_split == 2 || ctx->tune.matmul_rbm_split == 4) ks = (uint32_t)ctx->tune.matmul_rbm_split;
     R.ksplit = ks;
     const uint32_t NS = NW * ks, per = NS * SLOTS, hdr_dw = 8 + NS * 2;
-    std::vector<uint32_t> hdr((size_t)R.nb * hdr_dw, 0), rec;
+    std::vector<uint32_t> hdr((size_t)R.nb * hdr_dw, 0), rec, xrows;
     std::vector<float> w;
     rec.reserve((size_t)(E->total_nnz / 40 + (size_t)R.nb * NS * (TAILRECS + 8)) * RECDW);
     w.reserve(rec.capacity());
@@ -260,7 +268,7 @@ so_status so_rbmm_build(so_ctx *ctx, so_ellpack *E, const float *Wd, const uint3
                     const size_t wb = w.size();
                     for (uint32_t k = 0; k < SLOTS; ++k) {
                         const Part &pt = cls[s][g + k];
-                        rd[32 + k] = pt.j;
+                        xrows.push_back(pt.j);
                         for (uint32_t p = 0; p < MAXP; ++p)
                             rd[8 * k + p / 2] |= (IDXMODE | (p < s ? pt.pr[p].first : TRASH)) << (16 * (p % 2));
                         for (uint32_t p = 0; p < s; ++p) w.push_back(pt.pr[p].second);
@@ -274,6 +282,7 @@ so_status so_rbmm_build(so_ctx *ctx, so_ellpack *E, const float *Wd, const uint3
             for (uint32_t e = 0; e < TAILRECS; ++e) {             // what the loop requests past the stream's end
                 uint32_t rd[RECDW] = {0};
                 for (int k = 0; k < 32; ++k) rd[k] = (IDXMODE | TRASH) * 0x10001u;
+                xrows.resize(xrows.size() + SLOTS, 0);
                 rec.insert(rec.end(), rd, rd + RECDW);
                 w.resize(w.size() + RECDW, -0.0f);
             }
@@ -290,6 +299,9 @@ so_status so_rbmm_build(so_ctx *ctx, so_ellpack *E, const float *Wd, const uint3
     R.d_rec = (uint32_t *)p;
     if ((s = so_malloc(ctx, w.size() * 4, &p)) != SO_OK) return s;
     R.d_w = (float *)p;
+    if ((s = so_malloc(ctx, xrows.size() * 4, &p)) != SO_OK) return s;
+    R.d_xrows = (uint32_t *)p;
+    if ((s = so_h2d(ctx, R.d_xrows, xrows.data(), xrows.size() * 4)) != SO_OK) return s;
     if ((s = so_h2d(ctx, R.d_hdr, hdr.data(), hdr.size() * 4)) != SO_OK) return s;
     if ((s = so_h2d(ctx, R.d_rec, rec.data(), rec.size() * 4)) != SO_OK) return s;
     return so_h2d(ctx, R.d_w, w.data(), w.size() * 4);
@@ -301,6 +313,7 @@ void so_rbmm_free(so_ellpack *E)
     if (R.d_hdr) (void)hipFree(R.d_hdr);
     if (R.d_rec) (void)hipFree(R.d_rec);
     if (R.d_w) (void)hipFree(R.d_w);
+    if (R.d_xrows) (void)hipFree(R.d_xrows);
     R = so_rbmm();
 }
 
@@ -335,6 +348,14 @@ so_status so_matmul_rbm_launch(so_ctx *ctx, const so_ellpack *E, const float *dX
             SO_HIP(hipMemsetAsync(ctx->mm_counters, 0, cb, ctx->stream));
             SO_HIP(hipStreamSynchronize(ctx->stream));
         }
+    }
+    if (R.pitch != C * 4u) {
+        // the handle's records are rewritten for this pitch (stream-ordered; launches of one handle with
+        // different C must not overlap on different streams)
+        so_rbmm &Rw = const_cast<so_ellpack *>(E)->rbmm;
+        const uint64_t words = R.nrec * 4;
+        rbmm_offsets_kernel<<<so_ceil_div(words, 256), 256, 0, ctx->stream>>>(Rw.d_rec, Rw.d_xrows, R.nrec, C * 4u);
+        Rw.pitch = C * 4u;
     }
     switch (act) {
     case SO_ACT_RELU:    return launch_rbm<SO_ACT_RELU>(ctx, E, dX, C, dBias, dY);

@@ -88,6 +88,8 @@ struct so_rbmm {
     uint32_t *d_hdr = nullptr;                    // per block: iterations per class (6 dwords + 2 spare), then per stream {first record, first class}
     uint32_t *d_rec = nullptr;
     float *d_w = nullptr;
+    uint32_t *d_xrows = nullptr;                  // [nrec][4]: the X rows of every record; the records hold row * pitch
+    uint32_t pitch = 0;                           // row pitch of X (bytes) the records' offsets are written for; 0: none yet
 };
 
 struct so_ellpack {
