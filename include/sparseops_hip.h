@@ -116,9 +116,12 @@ so_status so_h2d(so_ctx *ctx, void *dst, const void *src, size_t bytes); /* wait
 so_status so_d2h(so_ctx *ctx, void *dst, const void *src, size_t bytes); /* waits */
 so_status so_d2d(so_ctx *ctx, void *dst, const void *src, size_t bytes);
 so_status so_fill_zero(so_ctx *ctx, void *dptr, size_t bytes); /* fill kernel, graph-safe */
-/* Waits for the context's stream.  SO_ERR_HIP if a wave of an earlier launch gave up waiting for
- * its workgroup (the LDS-staged kernels synchronise through counters with a bounded wait instead of
- * hanging): the results of those launches are invalid. */
+/* Waits for the context's stream.  The LDS-staged kernels synchronise their waves through counters
+ * with a bounded wait instead of hanging; a wave that gives up counts itself in a status word of the
+ * context.  Every call that waits for the stream -- so_sync, so_h2d, so_d2h, so_timer_end and the
+ * encoder's read-backs -- reads that word with the wait (one 4-byte copy, only when such a kernel has
+ * been launched since the last look) and returns SO_ERR_HIP when it is set: the results of the
+ * launches since the last look are invalid.  The word is then cleared; the next wait reports SO_OK. */
 so_status so_sync(so_ctx *ctx);
 
 /* HIP-event stopwatch on the context's stream: begin records an event, end

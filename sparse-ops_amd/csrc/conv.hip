@@ -427,7 +427,7 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
         auto store_next = [&]() {
             if (stored) return;
             stored = true;
-            so_lds::wait(sync_base + 8u + ((t + 1u) & 1u) * 4u, 16u * ((t + 1u) / 2u));
+            so_lds::wait(sync_base + 8u + ((t + 1u) & 1u) * 4u, 16u * ((t + 1u) / 2u), a.ws);
             store_window((t + 1u) & 1u);
             so_lds::signal(sync_base + ((t + 1u) & 1u) * 4u, lane);
         };
@@ -520,7 +520,7 @@ void conv2d_window_kernel(const int4 *__restrict__ stream, const uint32_t *__res
         if (DRIFT && a.nbuf == 2) {
             store_next();
             so_lds::signal(sync_base + 8u + cur_buf * 4u, lane);                    // done reading this chunk's buffer
-            if (more) so_lds::wait(sync_base + (cur_buf ^ 1u) * 4u, 16u * ((t + 1u) / 2u + 1u));   // the next window is complete
+            if (more) so_lds::wait(sync_base + (cur_buf ^ 1u) * 4u, 16u * ((t + 1u) / 2u + 1u), a.ws);   // the next window is complete
         } else if (a.nbuf == 2) {
             if (more) store_window(cur_buf ^ 1u);
             __syncthreads();
@@ -629,6 +629,7 @@ so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, 
     a.sth = window_step(plan->g.kH, plan->g.stride_h); a.stw = window_step(plan->g.kW, plan->g.stride_w);
     a.sbh = window_subsample(plan->g.kH, plan->g.stride_h); a.sbw = window_subsample(plan->g.kW, plan->g.stride_w);
     window_pixel_order(a, LPP);
+    a.ws = so_lds::wait_status{ctx->tune.wait_spins >= 0 ? (uint32_t)ctx->tune.wait_spins : so_lds::kSyncSpins, ctx->d_wait_gave_up};
     const size_t lds = (size_t)a.nbuf * a.buf_f4 * 16 + so_lds::kSyncBytes;
     // a layout whose chunks were sized for a smaller batch tile than this batch's does not fit
     if (LPP > w.lpp && (lds > (size_t)ctx->max_lds_bytes || a.win_f4 > (uint32_t)kWinMaxPerThread * kWinThreads)) return SO_OK;
@@ -644,6 +645,7 @@ so_status window_launch(so_ctx *ctx, const so_conv_plan *plan, const float *dX, 
     case 2:  window_launch_act<2, (int)LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
     default: window_launch_act<1, (int)LPP>(ctx, plan, a, grid, lds, dX, B, dBias, dResid, dY, act); break;
     }
+    ctx->waits_pending = true;
     *done = true;
     return SO_OK;
 }
@@ -828,7 +830,6 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
 
 } // namespace
 
-uint32_t so_conv_wait_timeouts() { return so_lds::take_wait_timeouts(); }
 
 extern "C" so_status so_conv_plan_create(so_ctx *ctx, const so_ellpack *E, const so_conv_geom *g,
                                          so_conv_plan **out)

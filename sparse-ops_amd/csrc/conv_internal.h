@@ -2,6 +2,7 @@
 #pragma once
 
 #include "so_internal.h"
+#include "lds_sync.h"
 
 #include <algorithm>
 #include <vector>
@@ -68,6 +69,7 @@ struct WinArgs {
     uint32_t sth, stw;  // window pixels between neighbouring output pixels
     uint32_t sbh, sbw;  // input pixels between neighbouring window pixels
     uint32_t order[16]; // slot -> output pixel of the tile (ty * TW + tx), one byte per slot; see window_pixel_order
+    so_lds::wait_status ws;   // bounded waits on the progress counters
 };
 
 // Along an axis on which the kernel has a single tap, a strided convolution reads only every

@@ -548,6 +548,7 @@ so_status so_conv_rbm_launch(so_ctx *ctx, const so_conv_plan *plan, const float 
     a.sth = window_step(plan->g.kH, plan->g.stride_h); a.stw = window_step(plan->g.kW, plan->g.stride_w);
     a.sbh = window_subsample(plan->g.kH, plan->g.stride_h); a.sbw = window_subsample(plan->g.kW, plan->g.stride_w);
     window_pixel_order(a, LPP);
+    a.ws = so_lds::wait_status{0, nullptr};      // this kernel synchronises with barriers
     const size_t lds = (size_t)a.nbuf * a.buf_f4 * 16;
     // a layout whose chunks were sized for a smaller batch tile than this batch's does not fit
     if (LPP > w.lpp && (lds > (size_t)ctx->max_lds_bytes || a.win_f4 > (uint32_t)kRbmMaxPerThread * kWinThreads)) return SO_OK;

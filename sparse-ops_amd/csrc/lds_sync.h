@@ -13,7 +13,8 @@
 // wave's operations in order, so the add lands after the wave's stores.  Waits cannot form a cycle:
 // every wait is for events of an earlier phase.  The poll nevertheless gives up after kSyncSpins
 // tries (a tenth of a second, thousands of launches long), so that no wave can ever hang here; a
-// wave that gives up counts itself in g_wait_timeouts, which so_sync() reports as an error.
+// wave that gives up counts itself in the context's status word (so_wait_status, passed to the
+// kernel), which every entry point that waits for the stream reads and reports as an error.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -25,8 +26,12 @@ namespace so_lds {
 constexpr uint32_t kSyncSpins = 1u << 20;
 constexpr uint32_t kSyncBytes = 64;      // LDS the counters take (four are used)
 
-// Waits that ran out of tries since the last look (one copy per translation unit that includes this).
-static __device__ uint32_t g_wait_timeouts;
+// What a kernel needs for its bounded waits: the most polls of one wait (the context's, so that a test
+// can make every wait give up at once) and where a wave that gives up counts itself.
+struct wait_status {
+    uint32_t spins;
+    uint32_t *gave_up;
+};
 
 // LDS byte address of a pointer into LDS.
 __device__ __forceinline__ uint32_t lds_address(const void *p) { return (uint32_t)(uintptr_t)p; }
@@ -36,25 +41,15 @@ __device__ __forceinline__ void signal(uint32_t addr, uint32_t lane)
     if (lane == 0) asm volatile("ds_add_u32 %0, %1" : : "v"(addr), "v"(1u) : "memory");
 }
 
-__device__ __forceinline__ void wait(uint32_t addr, uint32_t target)
+__device__ __forceinline__ void wait(uint32_t addr, uint32_t target, const wait_status &ws)
 {
-    for (uint32_t spin = 0; spin < kSyncSpins; ++spin) {
+    for (uint32_t spin = 0; spin < ws.spins; ++spin) {
         uint32_t v;
         asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(addr) : "memory");
         if (__builtin_amdgcn_readfirstlane(v) >= target) return;
         __builtin_amdgcn_s_sleep(2);
     }
-    if ((threadIdx.x & 63u) == 0) atomicAdd(&g_wait_timeouts, 1u);
-}
-
-// Host side: this translation unit's count, set back to zero.
-static inline uint32_t take_wait_timeouts()
-{
-    uint32_t n = 0;
-    const uint32_t zero = 0;
-    if (hipMemcpyFromSymbol(&n, HIP_SYMBOL(g_wait_timeouts), sizeof n) != hipSuccess) return 0;
-    if (n) (void)hipMemcpyToSymbol(HIP_SYMBOL(g_wait_timeouts), &zero, sizeof zero);
-    return n;
+    if ((threadIdx.x & 63u) == 0) atomicAdd(ws.gave_up, 1u);
 }
 
 } // namespace so_lds

@@ -36,7 +36,7 @@ void ellpack_matmul_tiled_kernel(const so_tile_entry *__restrict__ entries, cons
                                  const uint32_t *__restrict__ quad_rows, uint32_t nquads, uint32_t ntiles,
                                  uint32_t n, const float *__restrict__ X, uint32_t C,
                                  const float *__restrict__ bias, float *__restrict__ Y,
-                                 uint32_t nslabs, uint32_t ngroups, bool group_major)
+                                 uint32_t nslabs, uint32_t ngroups, bool group_major, so_lds::wait_status ws)
 {
     constexpr uint32_t KT = so_tiled::kTileRows, ROWB = so_tiled::kSlabCols * 4, TILE = so_tiled::kTileBytes;
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -136,7 +136,7 @@ void ellpack_matmul_tiled_kernel(const so_tile_entry *__restrict__ entries, cons
         for (int c = 0; c < kMaxChunks; ++c) {
             if (c == 1 && more) {
                 // the wave's part of the next tile, once every wave has finished the tile before this one
-                so_lds::wait(sync_base + 8u + ((t + 1u) & 1u) * 4u, 16u * ((t + 1u) / 2u));
+                so_lds::wait(sync_base + 8u + ((t + 1u) & 1u) * 4u, 16u * ((t + 1u) / 2u), ws);
                 lstore((t + 1) & 1u);
                 so_lds::signal(sync_base + ((t + 1u) & 1u) * 4u, lane);
             }
@@ -147,7 +147,7 @@ void ellpack_matmul_tiled_kernel(const so_tile_entry *__restrict__ entries, cons
             so_dpp::tiled_chunk(base, e.w, e.off, cur.steps - 16u * c, acc);
         }
         so_lds::signal(sync_base + 8u + (t & 1u) * 4u, lane);                                     // done reading this tile's buffer
-        if (more) so_lds::wait(sync_base + ((t + 1u) & 1u) * 4u, 16u * ((t + 1u) / 2u + 1u));     // the next tile is complete
+        if (more) so_lds::wait(sync_base + ((t + 1u) & 1u) * 4u, 16u * ((t + 1u) / 2u + 1u), ws);     // the next tile is complete
         cur = nxt;
 #pragma unroll
         for (int c = 0; c < kMaxChunks; ++c) { ew[c] = nw[c]; eo[c] = no[c]; }
@@ -174,13 +174,13 @@ so_status launch_tiled(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32
     const uint32_t blocks = grpmajor ? so_ceil_div(ngroups, 8) * 8 * nslabs
                                      : (8 % nslabs == 0) ? so_ceil_div(ngroups, 8 / nslabs) * 8 : nslabs * ngroups;
     ellpack_matmul_tiled_kernel<ACT><<<blocks, kTiledWaves * 64, so_tiled::kLdsBytes, ctx->stream>>>(
-        T.d_entries, T.d_info, T.d_rows, T.nquads, T.ntiles, E->n, dX, C, dBias, dY, nslabs, ngroups, grpmajor);
+        T.d_entries, T.d_info, T.d_rows, T.nquads, T.ntiles, E->n, dX, C, dBias, dY, nslabs, ngroups, grpmajor,
+        so_lds::wait_status{ctx->tune.wait_spins >= 0 ? (uint32_t)ctx->tune.wait_spins : so_lds::kSyncSpins, ctx->d_wait_gave_up});
+    ctx->waits_pending = true;
     return SO_OK;
 }
 
 } // namespace
-
-uint32_t so_matmul_wait_timeouts() { return so_lds::take_wait_timeouts(); }
 
 so_status so_matmul_tiled_launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
                                  const float *dBias, float *dY, int act)

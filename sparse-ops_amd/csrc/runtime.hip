@@ -74,6 +74,7 @@ static void read_tuning(so_tuning &t)
     t.conv_tilepx = env_int("SPARSEOPS_CONV_TILEPX", 0);
     t.conv_vec = env_int("SPARSEOPS_CONV_VEC", 0);
     t.conv_rbm = env_int("SPARSEOPS_CONV_RBM", -1);
+    t.wait_spins = env_int("SPARSEOPS_WAIT_SPINS", -1);
 }
 
 extern "C" so_status so_tuning_reload(so_ctx *ctx)
@@ -116,8 +117,36 @@ extern "C" so_status so_init(int device, so_ctx **out)
         so_destroy(ctx);
         return SO_ERR_HIP;
     }
+    // the word in which waves that give up a bounded wait count themselves, and its pinned host copy
+    e = hipMalloc((void **)&ctx->d_wait_gave_up, 64);
+    if (e == hipSuccess) e = hipMemset(ctx->d_wait_gave_up, 0, 64);
+    if (e == hipSuccess) e = hipHostMalloc((void **)&ctx->h_wait_gave_up, 64, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        so_set_error("so_init: allocating the wait status word failed: %s", hipGetErrorString(e));
+        so_destroy(ctx);
+        return e == hipErrorOutOfMemory ? SO_ERR_OOM : SO_ERR_HIP;
+    }
+    *ctx->h_wait_gave_up = 0;
     *out = ctx;
     return SO_OK;
+}
+
+// Waits for the stream; when a kernel with bounded waits has run since the last look, its status word
+// comes back with the same wait (one 4-byte copy queued behind the work) and is cleared if it was set.
+so_status so_stream_wait(so_ctx *ctx, const char *who)
+{
+    const bool look = ctx->waits_pending;
+    if (look) SO_HIP(hipMemcpyAsync(ctx->h_wait_gave_up, ctx->d_wait_gave_up, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    SO_HIP(hipStreamSynchronize(ctx->stream));
+    if (!look) return SO_OK;
+    ctx->waits_pending = false;
+    const uint32_t gave_up = *ctx->h_wait_gave_up;
+    if (gave_up == 0) return SO_OK;
+    *ctx->h_wait_gave_up = 0;
+    SO_HIP(hipMemsetAsync(ctx->d_wait_gave_up, 0, sizeof(uint32_t), ctx->stream));
+    SO_HIP(hipStreamSynchronize(ctx->stream));
+    so_set_error("%s: %u waits on LDS progress counters gave up in earlier launches; the results of those launches are invalid", who, gave_up);
+    return SO_ERR_HIP;
 }
 
 extern "C" so_status so_destroy(so_ctx *ctx)
@@ -127,6 +156,8 @@ extern "C" so_status so_destroy(so_ctx *ctx)
     if (ctx->stream) { (void)hipStreamSynchronize(ctx->stream); (void)hipStreamDestroy(ctx->stream); }
     if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
     if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+    if (ctx->d_wait_gave_up) (void)hipFree(ctx->d_wait_gave_up);
+    if (ctx->h_wait_gave_up) (void)hipHostFree(ctx->h_wait_gave_up);
     if (ctx->mm_part) (void)hipFree(ctx->mm_part);
     if (ctx->mm_counters) (void)hipFree(ctx->mm_counters);
     delete ctx;
@@ -172,8 +203,7 @@ extern "C" so_status so_h2d(so_ctx *ctx, void *dst, const void *src, size_t byte
     SO_REQUIRE(dst && src, "so_h2d: null pointer");
     SO_REQUIRE(!ctx->capturing, "so_h2d: not allowed while a graph is being recorded");
     SO_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
-    SO_HIP(hipStreamSynchronize(ctx->stream));
-    return SO_OK;
+    return so_stream_wait(ctx, "so_h2d");
 }
 
 extern "C" so_status so_d2h(so_ctx *ctx, void *dst, const void *src, size_t bytes)
@@ -183,8 +213,7 @@ extern "C" so_status so_d2h(so_ctx *ctx, void *dst, const void *src, size_t byte
     SO_REQUIRE(dst && src, "so_d2h: null pointer");
     SO_REQUIRE(!ctx->capturing, "so_d2h: not allowed while a graph is being recorded");
     SO_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
-    SO_HIP(hipStreamSynchronize(ctx->stream));
-    return SO_OK;
+    return so_stream_wait(ctx, "so_d2h");
 }
 
 extern "C" so_status so_d2d(so_ctx *ctx, void *dst, const void *src, size_t bytes)
@@ -220,14 +249,8 @@ extern "C" so_status so_sync(so_ctx *ctx)
 {
     SO_REQUIRE(ctx != nullptr, "so_sync: ctx is null");
     SO_REQUIRE(!ctx->capturing, "so_sync: not allowed while a graph is being recorded");
-    SO_HIP(hipStreamSynchronize(ctx->stream));
     // a kernel whose waves gave up waiting for one another has produced garbage: say so
-    const uint32_t gave_up = so_conv_wait_timeouts() + so_matmul_wait_timeouts();
-    if (gave_up) {
-        so_set_error("so_sync: %u waits on LDS progress counters timed out in earlier launches; their results are invalid", gave_up);
-        return SO_ERR_HIP;
-    }
-    return SO_OK;
+    return so_stream_wait(ctx, "so_sync");
 }
 
 extern "C" so_status so_timer_begin(so_ctx *ctx)
@@ -243,9 +266,9 @@ extern "C" so_status so_timer_end(so_ctx *ctx, float *ms)
     SO_REQUIRE(ctx && ms, "so_timer_end: null argument");
     SO_REQUIRE(!ctx->capturing, "so_timer_end: not allowed while a graph is being recorded");
     SO_HIP(hipEventRecord(ctx->ev1, ctx->stream));
-    SO_HIP(hipEventSynchronize(ctx->ev1));
+    const so_status s = so_stream_wait(ctx, "so_timer_end");
     SO_HIP(hipEventElapsedTime(ms, ctx->ev0, ctx->ev1));
-    return SO_OK;
+    return s;
 }
 
 // ---------------------------------------------------------------- launch graphs
@@ -286,6 +309,7 @@ extern "C" so_status so_graph_launch(so_ctx *ctx, so_graph *g)
     SO_REQUIRE(ctx && g && g->exec, "so_graph_launch: null argument");
     SO_REQUIRE(!ctx->capturing, "so_graph_launch: not allowed while recording");
     SO_HIP(hipGraphLaunch(g->exec, ctx->stream));
+    ctx->waits_pending = true;          // the graph may hold kernels with bounded waits
     return SO_OK;
 }
 
@@ -762,7 +786,8 @@ extern "C" so_status so_ellpack_encode_noalloc(so_ctx *ctx, const float *dDense,
     SO_REQUIRE(!ctx->capturing, "so_ellpack_encode_noalloc: r_out/total_nnz_out need a wait, which a graph recording forbids");
     uint32_t header[4] = {0, 0, 0, 0};
     SO_HIP(hipMemcpyAsync(header, ctx->static_scratch, sizeof header, hipMemcpyDeviceToHost, ctx->stream));
-    SO_HIP(hipStreamSynchronize(ctx->stream));
+    const so_status waited = so_stream_wait(ctx, "so_ellpack_encode_noalloc");
+    if (waited != SO_OK) return waited;
     if (r_out) *r_out = header[0];
     if (total_nnz_out) *total_nnz_out = (uint64_t)header[1] | ((uint64_t)header[2] << 32);
     SO_REQUIRE(header[0] <= r_cap, "so_ellpack_encode_noalloc: the longest row has %u nonzeros, dWd/dIdx hold %u per row (nothing was packed)",

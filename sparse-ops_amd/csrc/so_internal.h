@@ -22,6 +22,7 @@ struct so_tuning {
     int conv_cpw = 0;        // SPARSEOPS_CONV_CPW: most output channels per wave
     int conv_tilepx = 0;     // SPARSEOPS_CONV_TILEPX: most output pixels per tile
     int conv_vec = 0;        // SPARSEOPS_CONV_VEC: most batch entries per lane in the gather kernel
+    int wait_spins = -1;     // SPARSEOPS_WAIT_SPINS: most polls of a bounded wait on LDS progress counters (0: every wait gives up at once; tests)
     int conv_rbm = -1;       // SPARSEOPS_CONV_RBM: 0 forbids the row-block-merged kernel on plans that carry its streams
 };
 
@@ -34,6 +35,11 @@ struct so_ctx {
     bool capturing = false;
     void *static_scratch = nullptr;   // this device's address of the library's static scratch array (so_ellpack_encode_noalloc)
     // workspace of the row-block-merged matmul (csrc/matmul_rbm.hip): partial tiles of the workgroups that share a tile, a counter per tile
+    // Bounded waits (csrc/lds_sync.h): a device word in which waves that gave up count themselves, its pinned
+    // host copy, and whether a kernel that waits that way has been launched since the word was last looked at.
+    uint32_t *d_wait_gave_up = nullptr;
+    uint32_t *h_wait_gave_up = nullptr;
+    bool waits_pending = false;
     float *mm_part = nullptr;
     size_t mm_part_bytes = 0;
     uint32_t *mm_counters = nullptr;
@@ -138,9 +144,9 @@ bool so_matmul_rbm_applies(const so_ctx *ctx, const so_ellpack *E, uint32_t C);
 so_status so_matmul_rbm_launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
                                const float *dBias, float *dY, int act);
 
-// Waits on LDS progress counters (csrc/lds_sync.h) that gave up since the last call; so_sync() reports them.
-uint32_t so_conv_wait_timeouts();
-uint32_t so_matmul_wait_timeouts();
+// Waits for the context's stream and then reports, as SO_ERR_HIP, bounded waits that gave up in kernels launched
+// since the last look (their results are invalid).  Every entry point that waits for the stream ends with this.
+so_status so_stream_wait(so_ctx *ctx, const char *who);
 
 // Kernels that ask for more than 48 KB of dynamic LDS must be told so once per device: this does
 // it the first time `kernel` is seen on the context's device (hipSuccess when already done).

@@ -403,3 +403,37 @@ def test_matmul_rows_not_in_ascending_column_order(ctx, oracle):
     E2 = datagen.encode_dense(sparse_matrix(rng, 64, 300, .5))
     E2.idx[5, 1] = E2.idx[5, 0]
     assert np.array_equal(gpu_matmul(ctx, E2, X[:300], b[:64], "none", TILED), oracle.matmul(as_oracle(E2), X[:300], b[:64]))
+
+
+def test_bounded_wait_give_up_is_reported(ctx, oracle):
+    """The LDS-staged kernels' waits on progress counters are bounded.  With the poll budget set to zero
+    (SPARSEOPS_WAIT_SPINS=0) every wait gives up at once: the kernel still runs to its end, the waves count
+    themselves in the context's status word, and the next call that waits for the stream fails with
+    SO_ERR_HIP; the word is cleared by that, and a normal launch afterwards gives the oracle's bits."""
+    rng = np.random.default_rng(99)
+    W = sparse_matrix(rng, 256, 1024, .9)
+    X = rng.standard_normal((1024, 64)).astype(np.float32)
+    b = rng.standard_normal(256).astype(np.float32)
+    E = datagen.encode_dense(W)
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, TILED)
+    dX, dY, dB = ctx.array(X), ctx.empty((256, 64)), ctx.array(b)
+    ctx.sync()
+    with ctx.tuning(SPARSEOPS_MATMUL_TILED="1", SPARSEOPS_WAIT_SPINS="0"):
+        ctx.matmul(dE, dX, 64, dB, dY)
+        with pytest.raises(hipabi.SoError) as err:
+            ctx.sync()
+        assert err.value.status == hipabi.SO_ERR_HIP and "gave up" in str(err.value)
+        ctx.sync()                                        # reported once, then cleared
+    with ctx.tuning(SPARSEOPS_MATMUL_TILED="1"):
+        ctx.matmul(dE, dX, 64, dB, dY)
+        Y = dY.download()                                 # so_d2h looks at the word too: no error now
+    assert np.array_equal(Y, oracle.matmul(as_oracle(E), X, b))
+    # the same through a read-back: so_d2h reports what so_sync would
+    with ctx.tuning(SPARSEOPS_MATMUL_TILED="1", SPARSEOPS_WAIT_SPINS="0"):
+        ctx.matmul(dE, dX, 64, dB, dY)
+        with pytest.raises(hipabi.SoError):
+            dY.download()
+    ctx.sync()
+    for a in (dX, dY, dB):
+        a.free()
+    dE.free()
