@@ -32,15 +32,17 @@ for _p in (os.path.join(ROOT, "sparse-ops_amd"), os.path.join(ROOT, "sparse-ops_
 import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
-VALU_FP32_PEAK_TF = 157.3    # MI355X vector fp32; plain v_fma_f32 reaches 107 of its 128 multiply-adds per clock and CU,
-                             # the DPP form the quad layout needs 58 (profiles/lds_valu_rates__probe.txt)
+VALU_FP32_PEAK_TF = 157.3    # MI355X vector fp32; plain v_fma_f32 reaches 107 of its 128 multiply-adds per clock and CU, the
+                             # register-indexed DPP form of the row-block-merged kernel 77 at three waves per SIMD, the DPP
+                             # form of the quad layout 58 (profiles/lds_valu_rates__probe.txt, profiles/indexed_fma_rates__probe.txt)
 LDS_OPERAND_PEAK_TF = 78.6   # 256 CUs x 256 B/clk of ds_read_b128 (measured 255) x 2.4 GHz / 4 B per multiply-add x 2 flop
 # HBM-side bytes per launch, per kernel: measured with two rocprofv3 --pmc runs (FETCH_SIZE,
 # WRITE_SIZE) scaled by a plain copy of known size and kept, keyed by kernel name and together with a
 # hash of the kernel's sources, in this table (written by sparse-ops_amd/bench/pmc_summary.py traffic).
 # A kernel that is not in the table, or whose sources have changed since, reports null.
 TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-HEADLINE_KERNEL = "ellpack_matmul_tiled_kernel<0>"
+HEADLINE_KERNEL = "ellpack_matmul_rbm_kernel<0>"
+TILED_KERNEL = "ellpack_matmul_tiled_kernel<0>"
 MATVEC_KERNELS = {"ellpack_matvec 16384x16384, 95% Bernoulli": ("matvec_rows_kernel", "matvec 16384^2 uniform"),
                   "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048": ("matvec_binned_kernel", "matvec 16384^2 zipf")}
 
@@ -113,7 +115,7 @@ def host_has_avx512f():
         return False
 
 
-def cpu_baseline_matmul(E, X, bias, y_gpu, budget_s=15.0):
+def cpu_baseline_matmul(E, X, bias, y_gpu, y_exact, budget_s=15.0):
     """The same matmul on the host cores: the reference's compiled kernel when it
     can run here, else the plain-C restatement.  1 warm-up, then the median of as
     many runs as fit the budget (at least 5, at most 50) -- the reference
@@ -178,8 +180,10 @@ def cpu_baseline_matmul(E, X, bias, y_gpu, budget_s=15.0):
         "ms_per_step": round(med * 1e3, 4), "ms_per_step_min": round(min(times) * 1e3, 4), "cpu_model": model,
         "avx512f": host_has_avx512f(),       # without it the reference takes its scalar path (src/ellpack_matmul.cpp:80-90)
         "nnz_gflops_by_threads": by_threads,
-        "gpu_bit_exact_vs_cpu": bool(np.array_equal(Ycpu, y_gpu)),
+        # the headline (row-block-merged) kernel sums in another order: fp32 round-off; the K-tiled kernel gives the CPU's bits
         "gpu_max_rel_err_vs_cpu": float(np.abs(Ycpu.astype(np.float64) - y_gpu).max() / np.abs(Ycpu).max()),
+        "gpu_bit_exact_vs_cpu": bool(np.array_equal(Ycpu, y_gpu)),
+        "gpu_tiled_kernel_bit_exact_vs_cpu": bool(np.array_equal(Ycpu, y_exact)),
     }
 
 
@@ -398,18 +402,22 @@ def main():
 
     E, X, bias = datagen.config3()
     C = X.shape[1]
-    # ROW is the encoder's layout; TILED adds the K-tiled copy that so_matmul's
-    # LDS-staged kernel consumes (same nonzeros, same order inside every row).
-    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, hipabi.LAYOUT_ROW | hipabi.LAYOUT_TILED)
+    # ROW is the encoder's layout; RBM adds the row-block-merged copy the fastest so_matmul kernel consumes
+    # (fp32 round-off accuracy); TILED the K-tiled copy of the LDS-staged kernel (the reference's bits).
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, hipabi.LAYOUT_ROW | hipabi.LAYOUT_RBM)
     dX, dB, dY = ctx.array(X), ctx.array(bias), ctx.empty((E.m, C))
     step = lambda: ctx.matmul(dE, dX, C, dB, dY, "none")
     wall, ev_ms = time_launches(ctx, step, args.steps, args.warmup)
-    group_us = time_groups(ctx, step, 20, max(1, args.steps // 20))
+    group_us = time_groups(ctx, step, 20, max(10, args.steps // 20))
     y_gpu = dY.download()
-    # the row-per-wave kernel on the plain ROW layout, for comparison
+    # the bit-exact kernels on the same operands, for comparison: K-tiled (LDS-staged) and row-per-wave
+    dE_tiled = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, hipabi.LAYOUT_ROW | hipabi.LAYOUT_TILED)
+    _, ev_ms_tiled = time_launches(ctx, lambda: ctx.matmul(dE_tiled, dX, C, dB, dY, "none"), max(40, args.steps // 2), 5)
+    y_tiled = dY.download()
+    dE_tiled.free()
     dE_row = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, hipabi.LAYOUT_ROW)
     _, ev_ms_row = time_launches(ctx, lambda: ctx.matmul(dE_row, dX, C, dB, dY, "none"), max(20, args.steps // 4), 5)
-    row_bits_equal = bool(np.array_equal(dY.download(), y_gpu))
+    row_bits_equal = bool(np.array_equal(dY.download(), y_tiled))
     dE_row.free()
     ms_per_step = wall / args.steps * 1e3
     flops = 2.0 * E.total_nnz * C
@@ -426,22 +434,24 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBS, 4), "traffic": measured_traffic(HEADLINE_KERNEL),
                      "kernel": HEADLINE_KERNEL, "kernel_us": round(ev_ms * 1e3, 2),
-                     # 20 event-bracketed groups of K/20 launches each, per launch
+                     # 20 event-bracketed groups of max(10, K/20) launches each, per launch
                      "kernel_us_median": round(statistics.median(group_us), 2), "kernel_us_min": round(min(group_us), 2),
                      "alg_bytes_per_launch": nbytes,
-                     "row_kernel_us": round(ev_ms_row * 1e3, 2), "row_kernel_same_bits": row_bits_equal,
+                     "tiled_kernel_us": round(ev_ms_tiled * 1e3, 2), "tiled_kernel": TILED_KERNEL,
+                     "row_kernel_us": round(ev_ms_row * 1e3, 2), "row_kernel_same_bits_as_tiled": row_bits_equal,
+                     "max_rel_diff_vs_tiled_kernel": float(np.abs(y_gpu.astype(np.float64) - y_tiled).max() / np.abs(y_tiled).max()),
                      "valu_fp32_frac_of_157.3TF": round(flops / (ev_ms * 1e-3) / 1e12 / VALU_FP32_PEAK_TF, 4),
-                     # every multiply-add needs a 4-byte X operand from LDS/L1 (no reuse in registers):
-                     # bytes at that level, and the fraction of what LDS can deliver (256 B/clk/CU)
+                     # without reuse in registers every multiply-add needs a 4-byte X operand from LDS / L1 (what the
+                     # row and K-tiled kernels move at that level); the row-block-merged kernel loads an X row segment
+                     # once per 128-row block
                      "gather_bytes": 8 * E.total_nnz + 4 * E.total_nnz * C + 4 * E.m * C,
-                     "lds_operand_frac_of_78.6TF": round(flops / (ev_ms * 1e-3) / 1e12 / LDS_OPERAND_PEAK_TF, 4),
                      "t_hbm_us": round(nbytes / (HBM_PEAK_GBS * 1e9) * 1e6, 2),
                      "t_valu_us": round(flops / (VALU_FP32_PEAK_TF * 1e12) * 1e6, 2),
-                     "t_lds_operands_us": round(flops / (LDS_OPERAND_PEAK_TF * 1e12) * 1e6, 2),
-                     "t_bound_over_t": round(max(nbytes / (HBM_PEAK_GBS * 1e9), flops / (LDS_OPERAND_PEAK_TF * 1e12)) / (ev_ms * 1e-3), 4),
-                     "binding_bound": "not HBM (t_hbm 2.7 us): LDS operand reads (10.9 us at 256 B/clk/CU) and LDS tile writes (5.6 us at the "
-                                      "measured 78 B/clk/CU), multiply-adds in DPP form at half the plain rate (19 us with padding and address adds), and "
-                                      "the waves of a workgroup waiting for one another between the 16 tile phases (a quarter of a phase)"},
+                     "t_bound_over_t": round(max(nbytes / (HBM_PEAK_GBS * 1e9), flops / (VALU_FP32_PEAK_TF * 1e12)) / (ev_ms * 1e-3), 4),
+                     "binding_bound": "not HBM (t_hbm 2.7 us): the multiply-adds themselves -- one register-indexed v_fmac_f32_dpp plus one "
+                                      "M0 write per nonzero and 64 columns, 3.3 clk per SIMD at best (11 us at the 2.1 GHz the chip holds "
+                                      "under this load) -- then the sums of the 12 x 2 partial tiles per output tile (LDS, then memory) and "
+                                      "the launch's start-up; see DESIGN.md section 4"},
     }
     if args.calibrate_copy:
         # A plain copy of known size (act_kernel<NONE>: reads N floats, writes N floats)
@@ -457,7 +467,7 @@ def main():
         dst.free()
     if not args.no_cpu:
         log("timing the host-CPU baseline ...")
-        result["cpu_baseline"] = cpu_baseline_matmul(E, X, bias, y_gpu)
+        result["cpu_baseline"] = cpu_baseline_matmul(E, X, bias, y_gpu, y_tiled)
     else:
         result["cpu_baseline"] = None
     if not args.no_extras:

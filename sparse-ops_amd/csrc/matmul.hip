@@ -275,6 +275,13 @@ so_status launch_shared_gather(so_ctx *ctx, const so_ellpack *E, const float *dX
 
 } // namespace
 
+extern "C" so_status so_matmul_reserve(so_ctx *ctx, const so_ellpack *E, uint32_t C)
+{
+    SO_REQUIRE(ctx && E, "so_matmul_reserve: null argument");
+    if (E->m == 0 || C == 0 || !so_matmul_rbm_applies(ctx, E, C)) return SO_OK;
+    return so_matmul_rbm_reserve(ctx, E, C);
+}
+
 extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
                                const float *dBias, float *dY, int act)
 {

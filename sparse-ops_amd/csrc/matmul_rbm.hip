@@ -324,31 +324,37 @@ bool so_matmul_rbm_applies(const so_ctx *ctx, const so_ellpack *E, uint32_t C)
     return (size_t)ctx->max_lds_bytes >= LDS_BYTES;
 }
 
+// Grows the context's workspace (the partial tiles of the workgroups that share a tile, a counter per tile)
+// to what a launch of E with C dense columns needs.  Never while a graph is being recorded.
+so_status so_matmul_rbm_reserve(so_ctx *ctx, const so_ellpack *E, uint32_t C)
+{
+    const so_rbmm &R = E->rbmm;
+    const uint64_t tiles = (uint64_t)R.nb * so_ceil_div(C, 64);
+    SO_REQUIRE(tiles * R.ksplit < (1ull << 28), "so_matmul: %u x %u output is too large for one launch", E->m, C);
+    if (R.ksplit == 1) return SO_OK;
+    const size_t need_part = (size_t)tiles * R.ksplit * RB * 64 * sizeof(float), need_cnt = (size_t)tiles * sizeof(uint32_t);
+    if (need_part <= ctx->mm_part_bytes && need_cnt <= ctx->mm_counter_bytes) return SO_OK;
+    SO_REQUIRE(!ctx->capturing, "so_matmul: the row-block-merged kernel's workspace must grow, which cannot be done while a graph is "
+                                "being recorded (call so_matmul_reserve, or launch this shape once, before recording)");
+    SO_HIP(hipStreamSynchronize(ctx->stream));
+    if (ctx->mm_part) { (void)hipFree(ctx->mm_part); ctx->mm_part = nullptr; ctx->mm_part_bytes = 0; }
+    if (ctx->mm_counters) { (void)hipFree(ctx->mm_counters); ctx->mm_counters = nullptr; ctx->mm_counter_bytes = 0; }
+    const size_t pb = need_part + need_part / 4, cb = std::max<size_t>(need_cnt * 2, 4096);
+    SO_HIP(hipMalloc((void **)&ctx->mm_part, pb));
+    ctx->mm_part_bytes = pb;
+    SO_HIP(hipMalloc((void **)&ctx->mm_counters, cb));
+    ctx->mm_counter_bytes = cb;
+    SO_HIP(hipMemsetAsync(ctx->mm_counters, 0, cb, ctx->stream));
+    SO_HIP(hipStreamSynchronize(ctx->stream));
+    return SO_OK;
+}
+
 so_status so_matmul_rbm_launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
                                const float *dBias, float *dY, int act)
 {
     const so_rbmm &R = E->rbmm;
-    const uint32_t nslabs = so_ceil_div(C, 64);
-    const uint64_t tiles = (uint64_t)R.nb * nslabs;
-    SO_REQUIRE(tiles * R.ksplit < (1ull << 28), "so_matmul: %u x %u output is too large for one launch", E->m, C);
-    if (R.ksplit > 1) {
-        // workspace of the context: the partial tiles and one counter per tile; grown here, never while recording
-        const size_t need_part = (size_t)tiles * R.ksplit * RB * 64 * sizeof(float), need_cnt = (size_t)tiles * sizeof(uint32_t);
-        if (need_part > ctx->mm_part_bytes || need_cnt > ctx->mm_counter_bytes) {
-            SO_REQUIRE(!ctx->capturing, "so_matmul: the RBM kernel's workspace must grow, which cannot be done while a graph is being recorded "
-                                        "(launch this shape once before recording)");
-            SO_HIP(hipStreamSynchronize(ctx->stream));
-            if (ctx->mm_part) { (void)hipFree(ctx->mm_part); ctx->mm_part = nullptr; ctx->mm_part_bytes = 0; }
-            if (ctx->mm_counters) { (void)hipFree(ctx->mm_counters); ctx->mm_counters = nullptr; ctx->mm_counter_bytes = 0; }
-            const size_t pb = need_part + need_part / 4, cb = std::max<size_t>(need_cnt * 2, 4096);
-            SO_HIP(hipMalloc((void **)&ctx->mm_part, pb));
-            ctx->mm_part_bytes = pb;
-            SO_HIP(hipMalloc((void **)&ctx->mm_counters, cb));
-            ctx->mm_counter_bytes = cb;
-            SO_HIP(hipMemsetAsync(ctx->mm_counters, 0, cb, ctx->stream));
-            SO_HIP(hipStreamSynchronize(ctx->stream));
-        }
-    }
+    const so_status rs = so_matmul_rbm_reserve(ctx, E, C);
+    if (rs != SO_OK) return rs;
     if (R.pitch != C * 4u) {
         // the handle's records are rewritten for this pitch (stream-ordered; launches of one handle with
         // different C must not overlap on different streams)

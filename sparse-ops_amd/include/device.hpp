@@ -64,8 +64,9 @@ const so_ellpack *mirror(const Ellpack &E, int layouts);
 /// kernels take them per call.
 so_rbm *upload_rbm(const RBMPlan &plan);
 
-/// Device layouts to keep for Y = E * X with C dense columns (ROW, plus TILED
-/// where the LDS-staged kernel pays).
-int matmul_layouts(const Ellpack &E, uint32_t C);
+/// Device layouts to keep for Y = E * X with C dense columns: ROW, plus for large matrices and wide X
+/// either TILED (bit-identical to the reference) or, with `fast`, RBM (row-block-merged: the fastest
+/// kernel, results equal to fp32 round-off).
+int matmul_layouts(const Ellpack &E, uint32_t C, bool fast);
 
 } // namespace sparseops

@@ -20,7 +20,7 @@ LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS, LAYOUT_TILED, LAYOUT_RBM = 1, 2, 4, 8, 16
 SYMBOLS = (
     "so_device_count so_init so_destroy so_last_error so_device_info so_tuning_reload so_malloc so_free so_h2d so_d2h "
     "so_d2d so_fill_zero so_sync so_timer_begin so_timer_end so_ellpack_upload so_ellpack_free "
-    "so_ellpack_dims so_ellpack_download so_ellpack_decode so_ellpack_encode so_ellpack_encode_noalloc so_matmul so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
+    "so_ellpack_dims so_ellpack_download so_ellpack_decode so_ellpack_encode so_ellpack_encode_noalloc so_matmul so_matmul_reserve so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
     "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_copy_rows so_graph_begin so_graph_end "
     "so_graph_launch so_graph_free so_rbm_upload so_rbm_free so_rbm_dims so_conv_plan_set_rbm so_conv_plan_rbm_info").split()
 
@@ -81,6 +81,7 @@ def load_library(path=None):
         "so_ellpack_encode": [_vp, _vp, _u32, _u32, ct.POINTER(_vp)],
         "so_ellpack_encode_noalloc": [_vp, _vp, _u32, _u32, _u32, _vp, _vp, _vp, ct.POINTER(_u32), ct.POINTER(ct.c_uint64)],
         "so_matmul": [_vp, _vp, _vp, _u32, _vp, _vp, ct.c_int],
+        "so_matmul_reserve": [_vp, _vp, _u32],
         "so_matvec": [_vp, _vp, _vp, _vp, _vp, ct.c_int],
         "so_conv_plan_create": [_vp, _vp, ct.POINTER(ConvGeom), ct.POINTER(_vp)],
         "so_conv_plan_free": [_vp, _vp],
@@ -265,6 +266,9 @@ class Context:
 
     def matmul(self, E, dX, C, dBias, dY, act="none"):
         self._ck(self.lib.so_matmul(self.h, E.h, dX.ptr, C, dBias.ptr if dBias else None, dY.ptr, ACT[act]))
+
+    def matmul_reserve(self, E, C):
+        self._ck(self.lib.so_matmul_reserve(self.h, E.h, C))
 
     def matvec(self, E, dx, dBias, dy, layout=0):
         self._ck(self.lib.so_matvec(self.h, E.h, dx.ptr, dBias.ptr if dBias else None, dy.ptr, layout))

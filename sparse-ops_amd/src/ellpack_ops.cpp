@@ -20,14 +20,18 @@ Staging &staging()
 } // namespace
 
 namespace sparseops {
-// Device layouts worth keeping for Y = E * X with C dense columns: the K-tiled
-// copy (LDS-staged kernel) pays for large, reasonably filled matrices and wide X.
-int matmul_layouts(const Ellpack &E, uint32_t C)
+// Device layouts worth keeping for Y = E * X with C dense columns.  Large, reasonably filled
+// matrices and wide X pay for a second copy: the K-tiled one (LDS-staged kernel, the reference's
+// bits) or, with `fast`, the row-block-merged one (the fastest kernel; sums in another order,
+// accurate to fp32 round-off).
+int matmul_layouts(const Ellpack &E, uint32_t C, bool fast)
 {
     uint64_t total = 0;
     for (uint32_t c : E.nnz) total += c;
     const bool big = E.m >= 512 && E.n >= 512 && total >= 32ull * E.m;
-    return (big && C >= 64 && C % 4 == 0) ? (SO_LAYOUT_ROW | SO_LAYOUT_TILED) : SO_LAYOUT_ROW;
+    if (!big || C < 64) return SO_LAYOUT_ROW;
+    if (fast) return SO_LAYOUT_ROW | SO_LAYOUT_RBM;
+    return C % 4 == 0 ? (SO_LAYOUT_ROW | SO_LAYOUT_TILED) : SO_LAYOUT_ROW;
 }
 } // namespace sparseops
 
@@ -40,7 +44,7 @@ void matmul_host(const Ellpack &E, const float *X, uint32_t C, const float *bias
     so_ctx *ctx = context();
     std::lock_guard<std::mutex> lock(context_mutex());
     if (E.m == 0 || C == 0) return;
-    const so_ellpack *dE = mirror(E, matmul_layouts(E, C));
+    const so_ellpack *dE = mirror(E, matmul_layouts(E, C, false));     // host-pointer calls are PCIe-bound: keep the reference's bits
     Staging &st = staging();
     const std::size_t xbytes = std::size_t(E.n) * C * sizeof(float);
     const std::size_t ybytes = std::size_t(E.m) * C * sizeof(float);

@@ -41,8 +41,12 @@ void SparseOnnxModel::resize_buffers(uint32_t batch)
     if (pbatch != batch) M.stage_mid.reserve(widest * batch * sizeof(float));
     M.batch = batch;
     M.pbatch = pbatch;
-    for (const LayerPlan &L : M.layers)
+    for (const LayerPlan &L : M.layers) {
         if (L.conv) check(so_conv_plan_tune(ctx, L.conv, pbatch), "so_conv_plan_tune");
+        // whatever so_matmul would allocate at this batch is allocated now (run() allocates nothing, and a
+        // launch graph cannot be recorded across an allocation)
+        else if (L.op == Op::MatMul && L.dE) check(so_matmul_reserve(ctx, L.dE, pbatch), "so_matmul_reserve");
+    }
     if (M.use_graph && !M.layers.empty()) {
         check(so_graph_begin(ctx), "so_graph_begin");
         try {

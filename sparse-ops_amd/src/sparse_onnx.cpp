@@ -456,9 +456,13 @@ SparseOnnxModel::SparseOnnxModel(const std::string &onnx_path) : impl_(new Impl(
     // Weights, conv plans and biases into HBM.
     so_ctx *ctx = context();
     std::size_t bias_total = 0;
+    // Large fully connected layers run on the row-block-merged kernel (fp32 round-off accuracy, the fastest);
+    // SPARSEOPS_MATMUL_RBM=0 at load time keeps every layer on the kernels that give the reference's bits.
+    const char *rbm_env = std::getenv("SPARSEOPS_MATMUL_RBM");
+    const bool fast_fc = !(rbm_env && rbm_env[0] == '0');
     for (auto &p : pend) {
         if (p.plan.op != Op::MatMul && p.plan.op != Op::Conv) continue;
-        p.plan.dE = mirror(*p.plan.E, p.plan.op == Op::MatMul ? matmul_layouts(*p.plan.E, uint32_t(B0)) : SO_LAYOUT_ROW);
+        p.plan.dE = mirror(*p.plan.E, p.plan.op == Op::MatMul ? matmul_layouts(*p.plan.E, uint32_t(B0), fast_fc) : SO_LAYOUT_ROW);
         if (p.plan.op == Op::Conv) {
             check(so_conv_plan_create(ctx, p.plan.dE, &p.plan.cg, &p.plan.conv), "so_conv_plan_create");
             // The reference builds its row-block-merged plan for wide convolutions at load
