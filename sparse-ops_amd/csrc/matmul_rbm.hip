@@ -155,15 +155,27 @@ void ellpack_matmul_rbm_kernel(const uint32_t *__restrict__ hdr, const uint32_t 
     __syncthreads();
     if (*arrived != ksplit - 1) return;                      // the last workgroup of the tile to arrive finishes it
     if (tid == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+    // this wave's groups (w, w + 12, w + 24) of all partial tiles: every load is requested before the first is waited for
     const f32x4 *p = reinterpret_cast<const f32x4 *>(part) + (size_t)tile * ksplit * GROUPS * 64;
-    for (uint32_t g = wave; g < GROUPS; g += NW) {
-        f32x4 s;
-        asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(s) : "v"(p + g * 64 + lane) : "memory");
-        for (uint32_t k = 1; k < ksplit; ++k) {
-            f32x4 v;
-            asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p + ((size_t)k * GROUPS + g) * 64 + lane) : "memory");
-            s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
-        }
+    constexpr int kMine = (GROUPS + NW - 1) / NW;
+    f32x4 v[kMine][so_rbmm::kMaxSplit];
+#pragma unroll
+    for (int i = 0; i < kMine; ++i) {
+        const uint32_t g = wave + (uint32_t)i * NW;
+#pragma unroll
+        for (int k = 0; k < (int)so_rbmm::kMaxSplit; ++k)
+            if (g < GROUPS && (uint32_t)k < ksplit)
+                asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v[i][k]) : "v"(p + ((size_t)k * GROUPS + g) * 64 + lane) : "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+#pragma unroll
+    for (int i = 0; i < kMine; ++i) {
+        const uint32_t g = wave + (uint32_t)i * NW;
+        if (g >= GROUPS) break;
+        f32x4 s = v[i][0];
+#pragma unroll
+        for (int k = 1; k < (int)so_rbmm::kMaxSplit; ++k)
+            if ((uint32_t)k < ksplit) { s[0] += v[i][k][0]; s[1] += v[i][k][1]; s[2] += v[i][k][2]; s[3] += v[i][k][3]; }
         finish(g, s);
     }
 }
