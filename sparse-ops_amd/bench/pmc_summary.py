@@ -22,7 +22,7 @@ import statistics
 import sys
 
 ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-COPY_KERNEL = "act_kernel<0>"
+COPY_KERNEL = "act_kernel<0, false>"
 COPY_KIB = 262144.0      # bench.py --calibrate-copy: 256 MiB read, 256 MiB written per launch
 
 # Source files whose text decides a kernel's memory traffic: the table stores their hash, and
@@ -30,6 +30,8 @@ COPY_KIB = 262144.0      # bench.py --calibrate-copy: 256 MiB read, 256 MiB writ
 KERNEL_SOURCES = {
     "ellpack_matmul_tiled_kernel": ["sparse-ops_amd/csrc/matmul_tiled.hip", "sparse-ops_amd/csrc/dpp_steps.h",
                                     "sparse-ops_amd/csrc/lds_sync.h", "sparse-ops_amd/csrc/so_internal.h"],
+    "ellpack_matmul_rbm_kernel": ["sparse-ops_amd/csrc/matmul_rbm.hip", "sparse-ops_amd/csrc/gen_matmul_rbm_steps.py",
+                                  "sparse-ops_amd/csrc/so_internal.h"],
     "ellpack_matmul_kernel": ["sparse-ops_amd/csrc/matmul.hip", "sparse-ops_amd/csrc/so_internal.h"],
     "matvec_rows_kernel": ["sparse-ops_amd/csrc/matvec.hip"],
     "matvec_binned_kernel": ["sparse-ops_amd/csrc/matvec.hip"],

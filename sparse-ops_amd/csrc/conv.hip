@@ -971,8 +971,9 @@ static so_status conv2d_dispatch(so_ctx *ctx, const so_conv_plan *plan, const fl
     // 16, 8 or 4 (SPARSEOPS_CONV_WINDOW=1 forces it whenever possible, =0 forbids it: tuning and tests).
     const uint32_t lpp = window_lpp(B);
     if (plan->win.cc != 0 && lpp != 0 && (align & 15) == 0 && (uint64_t)plan->win.cc * g.H_in * g.W_in * B < (1ull << 31)) {
-        // a plan that carries the row-block-merged streams runs that kernel (SPARSEOPS_CONV_RBM=0 forbids it)
-        if (plan->rbm.d_sets && ctx->tune.conv_rbm != 0) {
+        // a plan that carries the row-block-merged streams runs that kernel (SPARSEOPS_CONV_RBM=0 forbids it).  It is an
+        // LDS-windowed kernel itself: SPARSEOPS_CONV_WINDOW=0 forbids it too, unless SPARSEOPS_CONV_RBM=1 asks for it.
+        if (plan->rbm.d_sets && ctx->tune.conv_rbm != 0 && (ctx->tune.conv_window != 0 || ctx->tune.conv_rbm == 1)) {
             bool done = false;
             const so_status s = so_conv_rbm_launch(ctx, plan, dX, B, dBias, dResid, dY, act, ctx->tune.conv_rbm == 1, &done);
             if (s != SO_OK) return s;

@@ -41,6 +41,11 @@ extern "C" so_status so_rbm_upload(so_ctx *ctx, uint32_t M, uint32_t N, uint32_t
     SO_REQUIRE(block_union[0] == 0 && colptr[0] == 0, "so_rbm_upload: block_union and colptr must start at 0");
     const uint32_t U = block_union[nblocks];
     SO_REQUIRE(U == 0 || krel != nullptr, "so_rbm_upload: krel is null");
+    // the pair arrays are read below: they must be there as soon as any union column claims a pair.  colptr has
+    // U + 1 entries by contract; what it says is checked entry by entry before it is used as an index.
+    bool any_pair = false;
+    for (uint32_t u = 0; u < U && !any_pair; ++u) any_pair = colptr[u + 1] != colptr[u];
+    SO_REQUIRE(!any_pair || (pair_row && pair_w), "so_rbm_upload: pair_row/pair_w is null");
     // every union column names a column of the matrix, columns ascend inside a block, every column
     // has at least one pair, the rows of a column ascend and lie inside the block
     for (uint32_t b = 0; b < nblocks; ++b) {

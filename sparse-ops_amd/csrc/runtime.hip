@@ -595,7 +595,7 @@ namespace {
 constexpr uint32_t kEncodeRowsPerBlock = 16;      // 4 waves x 4 rows
 constexpr uint32_t kEncodeMaxBlocks = 65536;      // workgroups whose partials the static scratch array holds
 constexpr uint32_t kEncodeHeaderBytes = 256;
-constexpr uint32_t kEncodeMaxCols = 1u << 28;     // 16 rows of that many columns still count in 32 bits
+constexpr uint32_t kEncodeMaxCols = (1u << 28) - 1;     // the 16 rows of a workgroup, all dense, still count in 32 bits
 constexpr size_t kEncodeScratchBytes = kEncodeHeaderBytes + (size_t)kEncodeMaxBlocks * sizeof(uint2);
 static_assert(kEncodeScratchBytes <= kStaticScratchBytes, "the static scratch array holds the encoder's partials");
 

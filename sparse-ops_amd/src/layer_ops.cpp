@@ -22,6 +22,14 @@ void act_inplace(int act, float *data, std::size_t len)
     check(so_d2h(ctx, data, buf.get(), len * sizeof(float)), "so_d2h");
 }
 
+bool rows_ascend(const Ellpack &E)
+{
+    for (uint32_t i = 0; i < E.m; ++i)
+        for (uint32_t k = 1; k < E.nnz[i]; ++k)
+            if (E.idx[std::size_t(i) * E.r + k] <= E.idx[std::size_t(i) * E.r + k - 1]) return false;
+    return true;
+}
+
 // The convolution on [C][H][W][B] host buffers.
 void conv_pf(const ConvAttr &c, const float *src_pf, uint32_t B, float *dst_pf)
 {
@@ -40,7 +48,10 @@ void conv_pf(const ConvAttr &c, const float *src_pf, uint32_t B, float *dst_pf)
         ~Cleanup() { if (plan) (void)so_conv_plan_free(ctx, plan); if (rbm) (void)so_rbm_free(ctx, rbm); }
     } cleanup{ctx, plan, rbm};
     if (B % 4 == 0) check(so_conv_plan_tune(ctx, plan, B), "so_conv_plan_tune");
-    if (c.use_rbm && !c.rbm.blocks.empty()) {
+    // The row-block-merged kernel takes blocks of at most 8 rows whose pairs ascend (what build_rbm_from_ellpack
+    // makes of rows with ascending columns); any other plan -- the reference's kernel allows blocks of up to 16
+    // rows, and a hand-filled matrix may have unordered rows -- runs on the per-row kernels: same result, same bits.
+    if (c.use_rbm && !c.rbm.blocks.empty() && c.rbm.Ct_max <= 8 && rows_ascend(c.E)) {
         rbm = upload_rbm(c.rbm);
         check(so_conv_plan_set_rbm(ctx, plan, rbm), "so_conv_plan_set_rbm");
     }

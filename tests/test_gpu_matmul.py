@@ -373,6 +373,12 @@ def test_device_encoder_degenerate(ctx):
     assert dE.r == 0 and np.array_equal(dE.decode(), np.zeros((6, 70), np.float32))
     dZ.free()
     dE.free()
+    # the column limit: 16 fully dense rows of 2^28 columns would wrap a workgroup's 32-bit nonzero count,
+    # so 2^28 columns are refused (argument check only: nothing is launched and the pointer is never read)
+    with pytest.raises(hipabi.SoError) as err:
+        h = hipabi.ct.c_void_p()
+        ctx._ck(ctx.lib.so_ellpack_encode(ctx.h, hipabi.ct.c_void_p(16), 1, 1 << 28, hipabi.ct.byref(h)))
+    assert err.value.status == hipabi.SO_ERR_INVALID and "columns" in str(err.value)
 
 
 def _shuffle_slots(E, rng):
