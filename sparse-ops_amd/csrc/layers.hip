@@ -102,11 +102,35 @@ void gap_kernel(uint32_t C, uint32_t HW, const float *__restrict__ X, uint32_t B
     }
 }
 
+// applyAdd (src/layers/add.cpp:9-76).  D may be A or B.  Aligned operands: 16 bytes per lane, chunks of 16 KB per
+// workgroup and operand, all eight loads of a lane requested before the first sum, non-temporal stores.
 __global__ __launch_bounds__(kBlock)
-void add_kernel(const float *__restrict__ A, const float *__restrict__ Bv, size_t len, float *D)
+void add_kernel(const float *A, const float *Bv, size_t len, float *D)
 {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    constexpr int U = 4;
+    constexpr size_t kChunk = (size_t)U * kBlock;
+    size_t done = 0;
+    if ((((uintptr_t)A | (uintptr_t)Bv | (uintptr_t)D) & 15u) == 0) {
+        const size_t nchunks = len / (4 * kChunk);
+        const f4 *A4 = reinterpret_cast<const f4 *>(A), *B4 = reinterpret_cast<const f4 *>(Bv);
+        f4 *D4 = reinterpret_cast<f4 *>(D);
+        for (size_t c = blockIdx.x; c < nchunks; c += gridDim.x) {
+            const size_t i = c * kChunk + threadIdx.x;
+            f4 a[U], b[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) { a[u] = A4[i + (size_t)u * kBlock]; b[u] = B4[i + (size_t)u * kBlock]; }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                f4 r;
+                r[0] = a[u][0] + b[u][0]; r[1] = a[u][1] + b[u][1]; r[2] = a[u][2] + b[u][2]; r[3] = a[u][3] + b[u][3];
+                __builtin_nontemporal_store(r, D4 + i + (size_t)u * kBlock);
+            }
+        }
+        done = nchunks * 4 * kChunk;
+    }
     const size_t stride = (size_t)gridDim.x * kBlock;
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < len; i += stride) D[i] = A[i] + Bv[i];
+    for (size_t i = done + (size_t)blockIdx.x * kBlock + threadIdx.x; i < len; i += stride) D[i] = A[i] + Bv[i];
 }
 
 // Streams X through the activation into Y (Y may be X).  Aligned operands go in chunks of 32 KB per workgroup:
@@ -212,7 +236,9 @@ extern "C" so_status so_add(so_ctx *ctx, const float *dA, const float *dB, size_
     SO_REQUIRE(ctx != nullptr, "so_add: ctx is null");
     if (len == 0) return SO_OK;
     SO_REQUIRE(dA && dB && dD, "so_add: null tensor");
-    add_kernel<<<blocks_for(ctx, len), kBlock, 0, ctx->stream>>>(dA, dB, len, dD);
+    // one workgroup per 16 KB chunk of each operand
+    const uint32_t blocks = (uint32_t)std::max<uint64_t>(1, std::min<uint64_t>((len + 4095) / 4096, 1u << 20));
+    add_kernel<<<blocks, kBlock, 0, ctx->stream>>>(dA, dB, len, dD);
     SO_LAUNCH_CHECK();
     return SO_OK;
 }

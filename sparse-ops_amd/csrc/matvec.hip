@@ -174,49 +174,101 @@ void matvec_rows_kernel(const float *__restrict__ Wd, const uint32_t *__restrict
     }
 }
 
+// Rows of at most G*T nonzeros, G lanes per row.  Such a row is a chain of memory round trips and
+// nothing else, so all of a group's first row is requested before x is staged.
+template <bool XLDS, int G, int T>
+__device__ __forceinline__ void short_rows(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
+                                           const uint2 *__restrict__ rows, uint32_t count, uint32_t block, uint32_t blocks,
+                                           uint32_t r, const float *__restrict__ x, uint32_t n, float *lds_x,
+                                           const float *__restrict__ bias, float *__restrict__ y)
+{
+    const uint32_t sub = threadIdx.x % G;
+    const uint32_t stride = blocks * (kBlock / G);
+    uint32_t g = block * (kBlock / G) + threadIdx.x / G;
+    const uint2 e = g < count ? rows[g] : make_uint2(0u, 0u);
+    const uint64_t base = (uint64_t)e.x * r;
+    float w[T];
+    uint32_t c[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        const uint32_t j = sub + G * t;
+        w[t] = j < e.y ? Wd[base + j] : 0.0f;
+        c[t] = j < e.y ? idx[base + j] : 0u;
+    }
+    const float *xs = stage_x<XLDS>(x, n, lds_x);
+    if (g < count) {
+        float a = 0.0f;
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const float xv = sub + G * t < e.y ? xs[c[t]] : 0.0f;      // x may be null when nothing is stored
+            a = __builtin_fmaf(w[t], xv, a);
+        }
+        for (uint32_t j = sub + G * T; j < e.y; j += G) a = __builtin_fmaf(Wd[base + j], xs[idx[base + j]], a);
+        a = group_sum<G>(a);
+        if (sub == 0) y[e.x] = (bias ? bias[e.x] : 0.0f) + a;
+    }
+    for (g += stride; g < count; g += stride) {
+        const uint2 en = rows[g];
+        const float s = group_row_dot<G>(Wd, idx, (uint64_t)en.x * r, en.y, xs, sub);
+        if (sub == 0) y[en.x] = (bias ? bias[en.x] : 0.0f) + s;
+    }
+}
+
 struct BinArgs {
-    const uint32_t *rows64, *rows16, *rows4;   // row ids per length class
+    const uint2 *rows64, *rows16, *rows4;      // (row, nonzeros of the row) per length class
     uint32_t n64, n16, n4;                     // rows per class
     uint32_t b64, b16;                         // workgroups given to the 64- and 16-lane classes
 };
 
 template <bool XLDS>
-__global__ __launch_bounds__(kBlock)
-void matvec_binned_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
-                          const uint32_t *__restrict__ nnz, BinArgs ba, uint32_t r,
+__global__ __launch_bounds__(kBlock, 8)          // 64 registers: two workgroups per compute unit
+void matvec_binned_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx, BinArgs ba, uint32_t r,
                           const float *__restrict__ x, uint32_t n,
                           const float *__restrict__ bias, float *__restrict__ y)
 {
     extern __shared__ float lds_x[];
-    const float *xs = stage_x<XLDS>(x, n, lds_x);
     const uint32_t b = blockIdx.x;
     if (b < ba.b64) {
+        // A wave's first row (its only one unless the class has more rows than the launch has waves):
+        // where it is and how long comes in one load, issued before x is staged.  The row itself is
+        // requested after the staging: asked for earlier, it delays x (loads return to a wave in
+        // order) and with it the barrier; measured 1.3 us slower on the Zipf matrix.
         const uint32_t lane = threadIdx.x & 63u;
         const uint32_t stride = ba.b64 * kWavesPerBlock;
-        for (uint32_t g = b * kWavesPerBlock + (threadIdx.x >> 6); g < ba.n64; g += stride) {
-            const uint32_t row = ba.rows64[g];
-            const uint64_t beg = (uint64_t)row * r;
-            const float s = wave_row_dot(reinterpret_cast<const f32x4 *>(Wd), reinterpret_cast<const u32x4 *>(idx),
-                                         beg, beg + nnz[row], xs, lane);
-            if (lane == 0) y[row] = (bias ? bias[row] : 0.0f) + s;
+        const f32x4 *Wd4 = reinterpret_cast<const f32x4 *>(Wd);
+        const u32x4 *idx4 = reinterpret_cast<const u32x4 *>(idx);
+        uint32_t g = __builtin_amdgcn_readfirstlane(b * kWavesPerBlock + (threadIdx.x >> 6));
+        const uint2 e = g < ba.n64 ? ba.rows64[g] : make_uint2(0u, 0u);
+        const uint64_t beg = (uint64_t)e.x * r, end = beg + e.y;
+        const uint64_t q0 = (beg >> 2) + lane;
+        const float *xs = stage_x<XLDS>(x, n, lds_x);
+        RowLoads A;
+        if (e.y > 0) row_issue(Wd4, idx4, beg, end, q0, A);
+        if (g < ba.n64) {
+            float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+            if (e.y > 0) {
+                row_consume(A, beg, end, q0, xs, a0, a1, a2, a3);
+                const uint64_t qlast = (end - 1) >> 2;
+                for (uint64_t q = q0 + 256; q <= qlast; q += 256) {
+                    RowLoads L;
+                    row_issue(Wd4, idx4, beg, end, q, L);
+                    row_consume(L, beg, end, q, xs, a0, a1, a2, a3);
+                }
+            }
+            const float s = group_sum<64>((a0 + a1) + (a2 + a3));
+            if (lane == 0) y[e.x] = (bias ? bias[e.x] : 0.0f) + s;
+        }
+        for (g += stride; g < ba.n64; g += stride) {
+            const uint2 en = ba.rows64[g];
+            const uint64_t nbeg = (uint64_t)en.x * r;
+            const float s = wave_row_dot(Wd4, idx4, nbeg, nbeg + en.y, xs, lane);
+            if (lane == 0) y[en.x] = (bias ? bias[en.x] : 0.0f) + s;
         }
     } else if (b < ba.b64 + ba.b16) {
-        const uint32_t sub = threadIdx.x & 15u;
-        const uint32_t stride = ba.b16 * (kBlock / 16);
-        for (uint32_t g = (b - ba.b64) * (kBlock / 16) + (threadIdx.x >> 4); g < ba.n16; g += stride) {
-            const uint32_t row = ba.rows16[g];
-            const float s = group_row_dot<16>(Wd, idx, (uint64_t)row * r, nnz[row], xs, sub);
-            if (sub == 0) y[row] = (bias ? bias[row] : 0.0f) + s;
-        }
+        short_rows<XLDS, 16, 8>(Wd, idx, ba.rows16, ba.n16, b - ba.b64, ba.b16, r, x, n, lds_x, bias, y);
     } else {
-        const uint32_t sub = threadIdx.x & 3u;
-        const uint32_t b4 = gridDim.x - ba.b64 - ba.b16;
-        const uint32_t stride = b4 * (kBlock / 4);
-        for (uint32_t g = (b - ba.b64 - ba.b16) * (kBlock / 4) + (threadIdx.x >> 2); g < ba.n4; g += stride) {
-            const uint32_t row = ba.rows4[g];
-            const float s = group_row_dot<4>(Wd, idx, (uint64_t)row * r, nnz[row], xs, sub);
-            if (sub == 0) y[row] = (bias ? bias[row] : 0.0f) + s;
-        }
+        short_rows<XLDS, 4, 4>(Wd, idx, ba.rows4, ba.n4, b - ba.b64 - ba.b16, gridDim.x - ba.b64 - ba.b16, r, x, n,
+                               lds_x, bias, y);
     }
 }
 
@@ -308,19 +360,19 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
     } else {
         // One launch over the three length classes.  bins[] is ordered 4, 16, 64 lanes.
         BinArgs ba;
-        ba.rows4 = E->bins[0].d_rows;   ba.n4 = E->bins[0].count;
-        ba.rows16 = E->bins[1].d_rows;  ba.n16 = E->bins[1].count;
-        ba.rows64 = E->bins[2].d_rows;  ba.n64 = E->bins[2].count;
+        ba.rows4 = reinterpret_cast<const uint2 *>(E->bins[0].d_rows);   ba.n4 = E->bins[0].count;
+        ba.rows16 = reinterpret_cast<const uint2 *>(E->bins[1].d_rows);  ba.n16 = E->bins[1].count;
+        ba.rows64 = reinterpret_cast<const uint2 *>(E->bins[2].d_rows);  ba.n64 = E->bins[2].count;
         ba.b64 = std::min(so_ceil_div(ba.n64, kWavesPerBlock), 2u * cus);
         ba.b16 = std::min(so_ceil_div(ba.n16, kBlock / 16), std::max(1u, cus / 4));
         const uint32_t b4 = std::min(so_ceil_div(ba.n4, kBlock / 4), std::max(1u, cus / 4));
         const uint32_t blocks = ba.b64 + ba.b16 + b4;
         if (blocks == 0) return SO_OK;
         if (use_lds(ctx, matvec_binned_kernel<true>, E->n, E->total_nnz, blocks))
-            matvec_binned_kernel<true><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, ba, E->r,
+            matvec_binned_kernel<true><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, E->d_idx, ba, E->r,
                                                                              dx, E->n, dBias, dy);
         else
-            matvec_binned_kernel<false><<<blocks, kBlock, 0, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, ba, E->r,
+            matvec_binned_kernel<false><<<blocks, kBlock, 0, ctx->stream>>>(E->d_Wd, E->d_idx, ba, E->r,
                                                                             dx, E->n, dBias, dy);
     }
     SO_LAUNCH_CHECK();

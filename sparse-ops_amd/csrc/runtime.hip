@@ -528,7 +528,13 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
                              [&](uint32_t a, uint32_t c) { return nnz[a] > nnz[c]; });
             E->bins[b].group = group[b];
             E->bins[b].count = (uint32_t)rows[b].size();
-            if (!rows[b].empty()) s = upload_array(ctx, rows[b].data(), rows[b].size(), &E->bins[b].d_rows);
+            // (row, its length) pairs: a wave learns where its row is and how long in one load
+            std::vector<uint32_t> pairs(2 * rows[b].size());
+            for (size_t k = 0; k < rows[b].size(); ++k) {
+                pairs[2 * k] = rows[b][k];
+                pairs[2 * k + 1] = nnz[rows[b][k]];
+            }
+            if (!pairs.empty()) s = upload_array(ctx, pairs.data(), pairs.size(), &E->bins[b].d_rows);
         }
     }
 

@@ -53,7 +53,7 @@ struct so_ctx {
 struct so_bin {
     uint32_t group = 0;      // 4, 16 or 64 lanes per row
     uint32_t count = 0;      // rows in this class
-    uint32_t *d_rows = nullptr;
+    uint32_t *d_rows = nullptr;   // count pairs (row, nonzeros of the row), longest rows first
 };
 
 // K-tiled copy of the matrix for the LDS-staged matmul.  Rows are grouped in
