@@ -22,8 +22,9 @@ import statistics
 import sys
 
 ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-COPY_KERNEL = "act_kernel<0, false>"
-COPY_KIB = 262144.0      # bench.py --calibrate-copy: 256 MiB read, 256 MiB written per launch
+COPY_KERNEL = "act_kernel<0,true>"     # the streaming instantiation of the plain copy, as short_name() writes it
+COPY_KIB = 262144.0      # bench.py --calibrate-copy: 256 MiB read, 256 MiB written per launch (run it with
+                         # --skip-extra stream_copy --skip-extra stream_copy_256MiB: the same kernel at other sizes)
 
 # Source files whose text decides a kernel's memory traffic: the table stores their hash, and
 # bench.py reports a kernel's traffic only while the hash still matches.

@@ -73,10 +73,12 @@ void ellpack_matmul_rbm_kernel(const uint32_t *__restrict__ hdr, const uint32_t 
     extern __shared__ __attribute__((aligned(16))) float red[];
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // Workgroup ids go round the 8 XCDs: the nslabs x ksplit workgroups of a row block take
-    // consecutive ids on one XCD, so the block's records and weights reach that L2 once.
-    const uint32_t xcd = blockIdx.x & 7u, q = blockIdx.x >> 3, per = nslabs * ksplit;
-    const uint32_t slab = q % nslabs, kh = (q / nslabs) % ksplit, b = (q / per) * 8u + xcd;
+    // Workgroup ids go round the 8 XCDs.  An XCD works on one part of K only (part kh of every
+    // stream set covers a contiguous range of columns, so its L2 holds 1/ksplit of X), and the
+    // nslabs workgroups that walk the same records take consecutive ids on it, so the records and
+    // weights reach that L2 once.
+    const uint32_t xcd = blockIdx.x & 7u, q = blockIdx.x >> 3, groups = 8u / ksplit;
+    const uint32_t slab = q % nslabs, kh = xcd % ksplit, b = (q / nslabs) * groups + xcd / ksplit;
     if (b >= nb) return;
     const uint32_t hdr_dw = 8u + NW * ksplit * 2u;
     const uint32_t *h = hdr + (size_t)b * hdr_dw;
@@ -194,7 +196,7 @@ so_status launch_rbm(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t
     const so_rbmm &R = E->rbmm;
     SO_HIP(so_allow_big_lds(ctx, (const void *)ellpack_matmul_rbm_kernel<ACT>));
     const uint32_t nslabs = so_ceil_div(C, 64);
-    const uint32_t blocks = so_ceil_div(R.nb, 8) * 8 * nslabs * R.ksplit;
+    const uint32_t blocks = so_ceil_div(R.nb, 8 / R.ksplit) * 8 * nslabs;      // ksplit is 1, 2 or 4
     ellpack_matmul_rbm_kernel<ACT><<<blocks, NW * 64, LDS_BYTES, ctx->stream>>>(
         R.d_hdr, R.d_rec, R.d_w, R.nrec, E->m, E->n, R.nb, R.ksplit, dX, C, dBias, dY, nslabs, ctx->mm_part, ctx->mm_counters);
     return SO_OK;
@@ -254,6 +256,7 @@ so_status so_rbmm_build(so_ctx *ctx, so_ellpack *E, const float *Wd, const uint3
             for (auto &p : single[s]) L.push_back(std::move(p));
             for (auto &p : carry) { p.pr.push_back(pad_pair); L.push_back(std::move(p)); }
             carry.clear();
+            std::stable_sort(L.begin(), L.end(), [](const Part &a, const Part &c) { return a.j < c.j; });
             if (s < MAXP) {                                       // what does not fill a round of all streams moves up a class
                 const size_t keep = L.size() / per * per;
                 for (size_t e = keep; e < L.size(); ++e) carry.push_back(std::move(L[e]));
@@ -275,7 +278,9 @@ so_status so_rbmm_build(so_ctx *ctx, so_ellpack *E, const float *Wd, const uint3
             for (uint32_t v = 0; v < NCLASS; ++v) {
                 const uint32_t s = CMIN + (entry - CMIN + v) % NCLASS;
                 for (uint32_t it = 0; it < q[s]; ++it) {
-                    const size_t g = ((size_t)it * NS + st) * SLOTS;
+                    // the class's parts are in column order: the kh-th of ksplit equal ranges belongs to the
+                    // streams of part kh, dealt four per iteration over its NW streams
+                    const size_t g = (size_t)(st / NW) * (cls[s].size() / ks) + ((size_t)it * NW + st % NW) * SLOTS;
                     uint32_t rd[RECDW] = {0};
                     const size_t wb = w.size();
                     for (uint32_t k = 0; k < SLOTS; ++k) {
