@@ -280,6 +280,12 @@ so_status so_act(so_ctx *ctx, int act, const float *dX, size_t len, float *dY);
  * array to the kernels' [F x B] layout and back (the reference's Python tests
  * do this on the host with Fortran-order arrays, tests/full_test.py:77-88). */
 so_status so_transpose(so_ctx *ctx, const float *dSrc, uint32_t rows, uint32_t cols, float *dDst);
+/* dst[i2][i1][i0][:] = src[i0][i1][i2][:] for a [d0][d1][d2][inner] array: converts between the
+ * kernels' [C][H][W][B] layout and a Fortran-order (B, C, H, W) array, which is [W][H][C][B] in memory
+ * (what conv2d_rbm_fmajor_implicit and conv2d_tiled_im2col_fmajor take, include/conv_kernels.hpp:8-24;
+ * the reference converts inside those kernels, src/layers/conv_kernels.cpp:96-123). */
+so_status so_reverse_axes3(so_ctx *ctx, const float *dSrc, uint32_t d0, uint32_t d1, uint32_t d2,
+                           uint32_t inner, float *dDst);
 /* Copy a [rows x cols] matrix between buffers whose rows start src_stride / dst_stride floats
  * apart; with zero_fill the rest of every destination row (cols .. dst_stride) is set to zero.
  * No counterpart in the reference: the model runtime uses it to carry a batch inside buffers whose

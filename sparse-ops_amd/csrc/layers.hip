@@ -189,6 +189,23 @@ void transpose_kernel(const float *__restrict__ src, uint32_t rows, uint32_t col
         if (c0 + i < cols && r0 + tx < rows) dst[(size_t)(c0 + i) * rows + r0 + tx] = tile[tx][i];
 }
 
+// dst[i2][i1][i0][:] = src[i0][i1][i2][:], rows of `inner` floats.  A lane per destination float:
+// writes are contiguous, reads come in runs of `inner` floats.
+__global__ __launch_bounds__(kBlock)
+void reverse_axes3_kernel(const float *__restrict__ src, uint32_t d0, uint32_t d1, uint32_t d2, uint32_t inner,
+                          float *__restrict__ dst, size_t total)
+{
+    const size_t stride = (size_t)gridDim.x * kBlock;
+    for (size_t o = (size_t)blockIdx.x * kBlock + threadIdx.x; o < total; o += stride) {
+        const uint32_t e = (uint32_t)(o % inner);
+        size_t t = o / inner;
+        const uint32_t i0 = (uint32_t)(t % d0);
+        t /= d0;
+        const uint32_t i1 = (uint32_t)(t % d1), i2 = (uint32_t)(t / d1);
+        dst[o] = src[(((size_t)i0 * d1 + i1) * d2 + i2) * inner + e];
+    }
+}
+
 uint32_t blocks_for(const so_ctx *ctx, uint64_t work)
 {
     const uint64_t need = (work + kBlock - 1) / kBlock;
@@ -302,6 +319,18 @@ extern "C" so_status so_transpose(so_ctx *ctx, const float *dSrc, uint32_t rows,
     const dim3 grid(so_ceil_div(cols, 64), so_ceil_div(rows, 64));
     SO_REQUIRE(grid.y < 65536, "so_transpose: too many rows");
     transpose_kernel<<<grid, kBlock, 0, ctx->stream>>>(dSrc, rows, cols, dDst);
+    SO_LAUNCH_CHECK();
+    return SO_OK;
+}
+
+extern "C" so_status so_reverse_axes3(so_ctx *ctx, const float *dSrc, uint32_t d0, uint32_t d1, uint32_t d2, uint32_t inner,
+                                      float *dDst)
+{
+    SO_REQUIRE(ctx != nullptr, "so_reverse_axes3: ctx is null");
+    const size_t total = (size_t)d0 * d1 * d2 * inner;
+    if (total == 0) return SO_OK;
+    SO_REQUIRE(dSrc && dDst && dSrc != dDst, "so_reverse_axes3: null or aliased tensor");
+    reverse_axes3_kernel<<<blocks_for(ctx, total), kBlock, 0, ctx->stream>>>(dSrc, d0, d1, d2, inner, dDst, total);
     SO_LAUNCH_CHECK();
     return SO_OK;
 }

@@ -9,11 +9,14 @@
 //   conv2d_tiled_im2col_fmajor   the same Fortran layout
 //   conv2d_tiled_im2col_cmajor   C-order (B,C,H,W)
 //
-// The last three convert on the host on the way in and out.  Each call uploads the weights' device
-// copy if it is not resident yet (cached on c.E), builds a convolution plan, copies src in and dst
-// out: convenience entry points for callers that drive single layers; SparseOnnxModel keeps plans
-// and activations resident.  With c.use_rbm set and c.rbm built (build_rbm_from_ellpack) the
-// row-block-merged kernel is attached to the plan; the result has the same bits either way.
+// The last three convert on the GPU on the way in and out (a 2-D transpose for the C-order layout, a
+// reversal of the three outer axes for the Fortran one).  The first call on a ConvAttr uploads the
+// weights' device copy (cached on c.E), builds the convolution plan and, with c.use_rbm set and c.rbm
+// built (build_rbm_from_ellpack), the row-block-merged streams, and keeps them with the staging
+// buffers on c.device; a repeated call with the same batch only copies src in, launches, and copies
+// dst out -- it allocates nothing.  Convenience entry points for callers that drive single layers;
+// SparseOnnxModel keeps activations resident as well.  The result has the same bits with or without
+// the row-block-merged kernel.
 // (For stride_w != 1 the reference's patch-major and C-major variants advance the input column by 1
 // instead of stride_w, src/layers/conv_kernels.cpp:436-447, 304-313; these compute the convolution.)
 // Throw std::runtime_error when no HIP device is usable or the geometry is inconsistent.

@@ -55,6 +55,18 @@ struct EllpackMirror {
     ~EllpackMirror();
 };
 
+/// What a ConvAttr keeps on the GPU between calls of the conv2d_* entry points (ConvAttr::device).
+struct ConvMirror {
+    so_conv_plan *plan = nullptr;
+    so_rbm *rbm = nullptr;
+    const void *ellpack = nullptr;        // the EllpackMirror the plan was built from
+    uint32_t geom[14] = {0};              // so_conv_geom as built
+    uint32_t tuned_batch = 0;
+    bool with_rbm = false;
+    DeviceBuffer in, out, bias, staged;   // grow-only: a repeated call allocates nothing
+    ~ConvMirror();
+};
+
 /// Upload E once (or again if `layouts` asks for more than is resident) and
 /// return the device handle.
 const so_ellpack *mirror(const Ellpack &E, int layouts);

@@ -10,6 +10,8 @@
 #include "ellpack_encoder.hpp"
 #include "rbm_conv.hpp"
 
+namespace sparseops { struct ConvMirror; }
+
 struct MatMulAttr {
     Ellpack E;
     float *bias_ptr = nullptr;   // length E.m, or null
@@ -43,6 +45,13 @@ struct ConvAttr {
     bool fuse_relu = false;
     RBMPlan rbm{};               // used when use_rbm is set and the plan is non-empty
     bool use_rbm{false};
+
+    // Addition: what the conv2d_* entry points keep on the GPU for this layer between calls (the
+    // convolution plan, the uploaded row-block-merged streams, staging buffers).  Built on the first
+    // call and rebuilt when the geometry members, the batch, use_rbm or E's device copy change; after
+    // editing `rbm` in place, call invalidate_device().
+    mutable std::shared_ptr<sparseops::ConvMirror> device;
+    void invalidate_device() const { device.reset(); }
 
     explicit ConvAttr(Ellpack e) : E(std::move(e)) {}
 };

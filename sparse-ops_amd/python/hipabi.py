@@ -21,7 +21,7 @@ SYMBOLS = (
     "so_device_count so_init so_destroy so_last_error so_device_info so_tuning_reload so_malloc so_free so_h2d so_d2h "
     "so_d2d so_fill_zero so_sync so_timer_begin so_timer_end so_ellpack_upload so_ellpack_free "
     "so_ellpack_dims so_ellpack_download so_ellpack_decode so_ellpack_encode so_ellpack_encode_noalloc so_matmul so_matmul_reserve so_matvec so_conv_plan_create so_conv_plan_free so_conv_plan_window so_conv_plan_tune so_conv2d_add "
-    "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_copy_rows so_graph_begin so_graph_end "
+    "so_conv2d so_maxpool so_gap so_add so_act so_transpose so_reverse_axes3 so_copy_rows so_graph_begin so_graph_end "
     "so_graph_launch so_graph_free so_rbm_upload so_rbm_free so_rbm_dims so_conv_plan_set_rbm so_conv_plan_rbm_info").split()
 
 _vp = ct.c_void_p
@@ -94,6 +94,7 @@ def load_library(path=None):
         "so_add": [_vp, _vp, _vp, ct.c_size_t, _vp],
         "so_act": [_vp, ct.c_int, _vp, ct.c_size_t, _vp],
         "so_transpose": [_vp, _vp, _u32, _u32, _vp],
+        "so_reverse_axes3": [_vp, _vp, _u32, _u32, _u32, _u32, _vp],
         "so_copy_rows": [_vp, _vp, ct.c_size_t, _u32, _u32, _vp, ct.c_size_t, ct.c_int],
         "so_graph_begin": [_vp],
         "so_graph_end": [_vp, ct.POINTER(_vp)],
@@ -138,10 +139,21 @@ class DeviceArray:
         self.ctx._ck(self.ctx.lib.so_d2h(self.ctx.h, _ptr(out), self.ptr, self.nbytes))
         return out
 
+    def offset(self, elems):
+        """A view of the flattened array that starts `elems` elements in; it does not own the memory."""
+        total = self.nbytes // self.dtype.itemsize
+        assert 0 <= elems <= total
+        v = object.__new__(DeviceArray)
+        v.ctx, v.shape, v.dtype = self.ctx, (total - elems,), self.dtype
+        v.nbytes = (total - elems) * self.dtype.itemsize
+        v.ptr = self.ptr + elems * self.dtype.itemsize
+        v._view = True
+        return v
+
     def free(self):
-        if self.ptr:
+        if self.ptr and not getattr(self, "_view", False):
             self.ctx.lib.so_free(self.ctx.h, self.ptr)
-            self.ptr = None
+        self.ptr = None
 
 
 class DeviceEllpack:
@@ -344,6 +356,9 @@ class Context:
 
     def transpose(self, dSrc, rows, cols, dDst):
         self._ck(self.lib.so_transpose(self.h, dSrc.ptr, rows, cols, dDst.ptr))
+
+    def reverse_axes3(self, dSrc, d0, d1, d2, inner, dDst):
+        self._ck(self.lib.so_reverse_axes3(self.h, dSrc.ptr, d0, d1, d2, inner, dDst.ptr))
 
     def copy_rows(self, dSrc, src_stride, rows, cols, dDst, dst_stride, zero_fill=False):
         self._ck(self.lib.so_copy_rows(self.h, dSrc.ptr, src_stride, rows, cols, dDst.ptr, dst_stride, int(zero_fill)))

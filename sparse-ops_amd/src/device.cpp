@@ -80,6 +80,12 @@ EllpackMirror::~EllpackMirror()
     if (handle) so_ellpack_free(context(), handle);
 }
 
+ConvMirror::~ConvMirror()
+{
+    if (plan) (void)so_conv_plan_free(context(), plan);
+    if (rbm) (void)so_rbm_free(context(), rbm);
+}
+
 const so_ellpack *mirror(const Ellpack &E, int layouts)
 {
     layouts |= SO_LAYOUT_ROW;

@@ -171,6 +171,8 @@ int main(int argc, char **argv)
         std::fill(out.begin(), out.end(), NAN);
         conv2d_patchmajor_tiled(c, src.data(), B, out.data());
         check(std::memcmp(out.data(), ref.data(), out.size() * sizeof(float)) == 0, "conv2d_patchmajor_tiled with the RBM plan attached");
+        const void *state = c.device.get();      // plan, RBM streams and staging buffers, kept on the ConvAttr
+        check(state != nullptr, "ConvAttr keeps its device state");
         // the same tensors in the Fortran (B,C,H,W) and the C-order (B,C,H,W) layouts
         std::vector<float> srcF(src.size()), srcC(src.size()), outF(ref.size(), NAN), outC(ref.size(), NAN);
         for (uint32_t ci = 0; ci < Cin; ++ci)
@@ -203,6 +205,7 @@ int main(int argc, char **argv)
                         okF2 &= outF[b + size_t(B) * (co + size_t(Cout) * (h + size_t(Ho) * w))] == ref[((size_t(co) * Ho + h) * Wo + w) * B + b];
         check(okF2, "conv2d_tiled_im2col_fmajor bit-exact");
         check(okC, "conv2d_tiled_im2col_cmajor (C-order layout) bit-exact");
+        check(c.device.get() == state, "repeated conv2d_* calls reuse the layer's device state");
     }
 
     if (argc == 5) {

@@ -320,6 +320,42 @@ def test_gap_add_act_transpose(ctx, oracle):
         assert np.array_equal(dT.download(), S.T)
 
 
+def test_add_long_and_unaligned(ctx):
+    """so_add over lengths that span many 16 KB chunks plus a tail, on operands that start off a 16-byte
+    boundary, and in place: D = A + B bit for bit (src/layers/add.cpp:9-76)."""
+    rng = np.random.default_rng(31)
+    n = 1_000_003
+    A, Bv = rng.standard_normal(n + 8).astype(np.float32), rng.standard_normal(n + 8).astype(np.float32)
+    dA, dB, dD = ctx.array(A), ctx.array(Bv), ctx.empty((n + 8,))
+    for off, length in ((0, n), (1, n - 5), (3, 4097), (0, 1), (2, 3)):
+        ctx.fill_zero(dD)
+        ctx.add(dA.offset(off), dB.offset(off), length, dD.offset(off))
+        got = dD.download()
+        assert np.array_equal(got[off:off + length], A[off:off + length] + Bv[off:off + length])
+        assert not got[off + length:].any() and not got[:off].any()
+    ctx.add(dA, dB, n, dB)
+    assert np.array_equal(dB.download()[:n], A[:n] + Bv[:n])
+
+
+@pytest.mark.parametrize("dims", [(7, 5, 3, 32), (56, 56, 64, 4), (1, 1, 1, 1), (3, 2, 5, 33), (2, 9, 1, 7)])
+def test_reverse_axes3(ctx, dims):
+    """so_reverse_axes3: [d0][d1][d2][inner] -> [d2][d1][d0][inner], i.e. a Fortran-order (B,C,H,W) array
+    ([W][H][C][B] in memory, include/conv_kernels.hpp:8-24) to [C][H][W][B] and back."""
+    rng = np.random.default_rng(9)
+    S = rng.standard_normal(dims).astype(np.float32)
+    dS, dT, dR = ctx.array(S), ctx.empty((dims[2], dims[1], dims[0], dims[3])), ctx.empty(dims)
+    ctx.reverse_axes3(dS, dims[0], dims[1], dims[2], dims[3], dT)
+    T = dT.download()
+    assert np.array_equal(T, S.transpose(2, 1, 0, 3))
+    ctx.reverse_axes3(dT, dims[2], dims[1], dims[0], dims[3], dR)
+    assert np.array_equal(dR.download(), S)
+    # the Fortran-order reading: element (b, c, h, w) of a (B, C, H, W) array with d = (W, H, C, B)
+    F = np.asfortranarray(rng.standard_normal((dims[3], dims[2], dims[1], dims[0])).astype(np.float32))
+    dF = ctx.array(np.frombuffer(F.tobytes(order="F"), dtype=np.float32))
+    ctx.reverse_axes3(dF, dims[0], dims[1], dims[2], dims[3], dT)
+    assert np.array_equal(dT.download(), np.ascontiguousarray(F.transpose(1, 2, 3, 0)))
+
+
 def test_launch_graph_replays(ctx, oracle):
     """A recorded chain replays with the same bits as eager execution, several
     times, with eager work and synchronisation in between."""
