@@ -4,6 +4,8 @@
     python sparse-ops_amd/bench/pmc_summary.py counters <counter_collection.csv> [...more csv] [--kernels REGEX]
     # kernel durations of a --kernel-trace run (csv output):
     python sparse-ops_amd/bench/pmc_summary.py trace <kernel_trace.csv> [--kernels REGEX] [--skip N]
+    # the kernels of one forward pass of a layer chain, in launch order (averages over the passes found):
+    python sparse-ops_amd/bench/pmc_summary.py layers <kernel_trace.csv> --last gap_kernel
     # HBM-side bytes per launch from a FETCH_SIZE run and a WRITE_SIZE run, scaled by the plain copy
     # kernel of known size that `bench.py --calibrate-copy` launches, written into the table bench.py
     # reads `roofline.traffic` from:
@@ -107,6 +109,37 @@ def cmd_trace(a):
         print("(avg / median / min / max leave out each kernel's first %d calls)" % a.skip)
 
 
+def cmd_layers(a):
+    """A forward pass = the dispatches up to and including the one after each dispatch of the kernel
+    named by --last (a chain's second-to-last layer) whose grid is the largest seen for that kernel
+    (the largest batch); passes are as long as the most common distance between two such dispatches."""
+    with open(a.csv[0], newline="") as f:
+        rows = sorted(csv.DictReader(f), key=lambda r: int(r["Start_Timestamp"]))
+    names = [short_name(r["Kernel_Name"]) for r in rows]
+    grid = [int(r.get("Grid_Size") or r.get("Grid_Size_X") or 0) for r in rows]
+    marks = [i for i, k in enumerate(names) if k.split("<")[0] == a.last]
+    if not marks:
+        sys.exit("no dispatch of %s in the trace" % a.last)
+    big = max(grid[i] for i in marks)
+    marks = [i for i in marks if grid[i] == big and i + 1 < len(rows)]
+    gaps = collections.Counter(b - c for c, b in zip(marks, marks[1:]))
+    if not gaps:
+        sys.exit("fewer than two passes in the trace")
+    count = gaps.most_common(1)[0][0]
+    passes = [list(range(i + 2 - count, i + 2)) for i in marks if i + 2 - count >= 0]
+    ref = [names[j] for j in passes[-1]]
+    passes = [p for p in passes if [names[j] for j in p] == ref]
+    print("%d kernels per pass, %d passes with this sequence (grid of %s: %d work-items)" % (count, len(passes), a.last, big))
+    print("%3s %-44s %12s %10s %10s %10s" % ("#", "kernel", "grid", "avg us", "min us", "max us"))
+    total = 0.0
+    for pos in range(count):
+        d = [(int(rows[p[pos]]["End_Timestamp"]) - int(rows[p[pos]]["Start_Timestamp"])) / 1e3 for p in passes]
+        total += sum(d) / len(d)
+        print("%3d %-44s %12d %10.1f %10.1f %10.1f" % (pos + 1, ref[pos], grid[passes[-1][pos]], sum(d) / len(d), min(d), max(d)))
+    span = [(int(rows[p[-1]]["End_Timestamp"]) - int(rows[p[0]]["Start_Timestamp"])) / 1e3 for p in passes]
+    print("sum of the kernels %.1f us; first start to last end of a pass: avg %.1f us, min %.1f us" % (total, sum(span) / len(span), min(span)))
+
+
 def cmd_traffic(a):
     fetch = read_counters([a.csv[0]], None)
     write = read_counters([a.csv[1]], None)
@@ -166,14 +199,15 @@ def lookup_traffic(table_path, kernel, workload=None):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("mode", choices=["counters", "trace", "traffic"])
+    ap.add_argument("mode", choices=["counters", "trace", "layers", "traffic"])
     ap.add_argument("csv", nargs="+")
     ap.add_argument("--kernels", default=None, help="regular expression on the short kernel name")
     ap.add_argument("--skip", type=int, default=0, help="trace: calls to leave out of the averages (warm-up)")
+    ap.add_argument("--last", default="gap_kernel", help="layers: name of the chain's second-to-last kernel")
     ap.add_argument("--update", default=None, help="traffic: JSON table to update")
     ap.add_argument("--workload", default=None, help="traffic: key suffix when one kernel is measured on several workloads")
     a = ap.parse_args()
-    {"counters": cmd_counters, "trace": cmd_trace, "traffic": cmd_traffic}[a.mode](a)
+    {"counters": cmd_counters, "trace": cmd_trace, "layers": cmd_layers, "traffic": cmd_traffic}[a.mode](a)
 
 
 if __name__ == "__main__":
