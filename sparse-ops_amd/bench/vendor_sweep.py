@@ -34,13 +34,13 @@ def run(args):
 
 
 def summarize(label, rows):
-    ours = min(v[0] for k, v in rows.items() if k.startswith("Ellpack"))
+    ours = min((v[0], k) for k, v in rows.items() if k.startswith("Ellpack"))
     sparse = [(v[0], k) for k, v in rows.items() if k.startswith("rocSPARSE")]
     dense = [v[0] for k, v in rows.items() if k.startswith("rocBLAS")]
     worst = max(v[1] for v in rows.values())
     best_sparse = min(sparse) if sparse else (float("nan"), "-")
-    print("| %-44s | %8.1f | %8.1f (%s) | %8.1f | %.1e |" % (
-        label, ours, best_sparse[0], best_sparse[1].split("(")[-1].rstrip(")"), dense[0] if dense else float("nan"), worst))
+    print("| %-44s | %8.1f (%s) | %8.1f (%s) | %8.1f | %.1e |" % (
+        label, ours[0], ours[1].split("(")[-1].rstrip(")"), best_sparse[0], best_sparse[1].split("(")[-1].rstrip(")"), dense[0] if dense else float("nan"), worst))
     sys.stdout.flush()
 
 
@@ -50,7 +50,7 @@ def main():
     ap.add_argument("--quick", action="store_true", help="small shapes only")
     a = ap.parse_args()
     runs = ["--runs", str(a.runs)]
-    print("| case | so_matmul / so_matvec us | rocSPARSE CSR us (best algorithm) | rocBLAS dense us | max rel diff |")
+    print("| case | so_matmul / so_matvec us (fastest kernel) | rocSPARSE CSR us (best algorithm) | rocBLAS dense us | max rel diff |")
     print("|---|---|---|---|---|")
     sizes = [512] if a.quick else [512, 1024, 2048]
     for n in sizes:
