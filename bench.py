@@ -449,9 +449,9 @@ def main():
                      "t_valu_us": round(flops / (VALU_FP32_PEAK_TF * 1e12) * 1e6, 2),
                      "t_bound_over_t": round(max(nbytes / (HBM_PEAK_GBS * 1e9), flops / (VALU_FP32_PEAK_TF * 1e12)) / (ev_ms * 1e-3), 4),
                      "binding_bound": "not HBM (t_hbm 2.7 us): the multiply-adds themselves -- one register-indexed v_fmac_f32_dpp plus one "
-                                      "M0 write per nonzero and 64 columns, 3.3 clk per SIMD at best (11 us at the 2.1 GHz the chip holds "
-                                      "under this load) -- then the sums of the 12 x 2 partial tiles per output tile (LDS, then memory) and "
-                                      "the launch's start-up; see DESIGN.md section 4"},
+                                      "M0 write per nonzero and 64 columns, a dependent pair that takes a wave 10 clk: 3.4 clk per SIMD at the "
+                                      "kernel's 3 waves per SIMD, 10.7 us for the launch's 6.9 M pairs -- then waiting for the records' scalar "
+                                      "loads, the sums of the 12 x 2 partial tiles per output tile (LDS, then memory) and the launch's start-up"},
     }
     if args.calibrate_copy:
         # A plain copy of known size (act_kernel<NONE>: reads N floats, writes N floats)
