@@ -3,9 +3,8 @@
 // same flags (--M --N --C --sparsity --runs --seed --irregular), same data recipe
 // (N(0,1) values under an i.i.d. Bernoulli mask, optionally a dense last row; X ~ U(-1,1);
 // no bias; benchmark-mkl/common/data_gen.cpp:23-96), 1 warm-up then the median of --runs,
-// reported in microseconds.  Random numbers come from std::mt19937_64 through explicit
-// transforms (53-bit uniforms, Box-Muller normals): the standard library's distribution
-// classes may differ between implementations, these do not.  --ellpack-file <path> replaces
+// reported in microseconds.  The matrices come from data_gen.hpp, which Python reaches too
+// (sparseops_backend.benchmark_dense): one seed, one matrix on both sides.  --ellpack-file <path> replaces
 // the generated matrix by one written by python/datagen.py's save_ellpack (any of the
 // benchmark configurations), so the very same matrix runs here and in bench.py.  The comparators are the ROCm counterparts of the reference's:
 // rocSPARSE CSR SpMM / SpMV for MKL sparse, rocBLAS SGEMM / SGEMV for the dense BLAS, and
@@ -28,6 +27,7 @@
 #include <string>
 #include <vector>
 
+#include "data_gen.hpp"
 #include "sparseops_hip.h"
 
 #define HIPCK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { std::fprintf(stderr, "%s: %s\n", #x, hipGetErrorString(e_)); std::exit(2); } } while (0)
@@ -47,14 +47,6 @@ struct Host {
     std::vector<uint32_t> idx, nnz;
 };
 
-// Explicit transforms of the generator's 64-bit outputs.
-inline double uniform01(std::mt19937_64 &rng) { return double(rng() >> 11) * (1.0 / 9007199254740992.0); }   // [0, 1), 53 bits
-inline float normal01(std::mt19937_64 &rng)
-{
-    const double u1 = 1.0 - uniform01(rng), u2 = uniform01(rng);                                              // u1 in (0, 1]
-    return float(std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586476925 * u2));
-}
-
 // CSR and ELLPACK views of the dense matrix in h.W.
 void derive_formats(Host &h);
 
@@ -62,12 +54,7 @@ Host generate(int64_t M, int64_t N, double sparsity, uint64_t seed, bool irregul
 {
     Host h;
     h.M = M; h.N = N;
-    h.W.assign(size_t(M) * N, 0.0f);
-    std::mt19937_64 rng(seed);
-    const double keep = 1.0 - sparsity;
-    for (int64_t i = 0; i < M; ++i)
-        for (int64_t j = 0; j < N; ++j)
-            if ((irregular && i == M - 1) || uniform01(rng) < keep) h.W[size_t(i) * N + j] = normal01(rng);
+    h.W = sparseops_bench::dense_matrix(M, N, sparsity, seed, irregular);
     derive_formats(h);
     return h;
 }
@@ -227,11 +214,7 @@ int main(int argc, char **argv)
                 "Repetitions:     %d\nRNG seed:        %llu\nIrregular last row: %d\n\n",
                 matmul ? "MatMul" : "MatVec", (long long)M, (long long)N, C, sparsity, runs, (unsigned long long)seed, int(irregular));
 
-    std::vector<float> X(size_t(N) * C);
-    {
-        std::mt19937_64 rng(seed);
-        for (auto &v : X) v = float(2.0 * uniform01(rng) - 1.0);
-    }
+    const std::vector<float> X = sparseops_bench::dense_operand(size_t(N) * C, seed);
     const size_t nnz_total = h.values.size();
     std::printf("nnz %zu, ELLPACK r %u (padding %.2fx)\n\n", nnz_total, h.r, nnz_total ? double(M) * h.r / nnz_total : 0.0);
 

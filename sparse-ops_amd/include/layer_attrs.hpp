@@ -5,12 +5,22 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <memory>
+#include <string>
+#include <variant>
 #include <vector>
 
 #include "ellpack_encoder.hpp"
 #include "rbm_conv.hpp"
 
 namespace sparseops { struct ConvMirror; }
+
+// What kind of node a layer is, and which operator exactly (include/sparse_onnx.hpp:30-47).
+enum class LayerType { MatMul, Activation, Elementwise, Pool, Reshape, Conv };
+enum class LayerOp { MatMul, Relu, Sigmoid, Tanh, Add, MaxPool, GlobalAveragePool, Flatten, Conv };
+// Memory order of a 4-D activation (include/sparse_onnx.hpp:49): Fortran-order (B,C,H,W), C-order
+// (B,C,H,W), or [C][H][W][B]; the conv2d_* entry points of conv_kernels.hpp take one each.
+enum class DataLayout : uint8_t { BFastFortran, NCHW_C, PatchMajor };
 
 struct MatMulAttr {
     Ellpack E;
@@ -68,3 +78,23 @@ struct PoolAttr {
 struct FlattenAttr { int axis; };
 struct AddAttr {};
 struct ActAttr {};
+
+// One node of a layer chain as a caller may assemble it (include/sparse_onnx.hpp:113-131): the
+// payload for its kind plus the names of the graph values it reads and writes.
+using LayerAttr = std::variant<MatMulAttr, ConvAttr, PoolAttr, FlattenAttr, AddAttr, ActAttr>;
+
+struct Layer {
+    LayerType type;
+    LayerOp op;
+    LayerAttr attr;
+    std::vector<std::string> inputs;
+    std::vector<std::string> outputs;
+};
+
+// A layer's result as the reference's per-layer helpers hand it on (include/sparse_onnx.hpp:134-138):
+// `features` rows of the batch; `owned` says whether the receiver frees `data`.
+struct RunResult {
+    float *data;
+    uint32_t features;
+    bool owned;
+};

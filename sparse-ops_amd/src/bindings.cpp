@@ -8,6 +8,7 @@
 
 #include <cstring>
 
+#include "../bench/data_gen.hpp"
 #include "device.hpp"
 #include "ellpack_encoder.hpp"
 #include "ellpack_matmul.hpp"
@@ -188,6 +189,23 @@ PYBIND11_MODULE(sparseops_backend, mod)
     }, py::arg("E"), py::arg("bias") = py::none(), py::arg("Ct_max") = 8,
        "Row-block-merged re-encoding of an ELLPACK matrix (blocks of Ct_max rows, union columns, (row, weight) pairs)");
 
+    // The benchmark harness's generator (bench/data_gen.hpp; the reference's recipe,
+    // benchmark-mkl/common/data_gen.cpp:23-96): what bench_vendor runs for the same arguments.
+    mod.def("benchmark_dense", [](int64_t M, int64_t N, double sparsity, uint64_t seed, bool irregular) {
+        if (M < 0 || N < 0 || !(sparsity >= 0.0 && sparsity <= 1.0)) throw std::runtime_error("benchmark_dense: bad arguments");
+        const std::vector<float> W = sparseops_bench::dense_matrix(M, N, sparsity, seed, irregular);
+        py::array_t<float> out({py::ssize_t(M), py::ssize_t(N)});
+        std::copy(W.begin(), W.end(), out.mutable_data());
+        return out;
+    }, py::arg("M"), py::arg("N"), py::arg("sparsity"), py::arg("seed") = 42, py::arg("irregular") = false,
+       "Dense (M, N) float32 matrix of the benchmark recipe: Bernoulli(1 - sparsity) mask over N(0, 1) values");
+    mod.def("benchmark_operand", [](py::ssize_t rows, py::ssize_t cols, uint64_t seed) {
+        if (rows < 0 || cols < 0) throw std::runtime_error("benchmark_operand: bad arguments");
+        const std::vector<float> X = sparseops_bench::dense_operand(std::size_t(rows) * std::size_t(cols), seed);
+        py::array_t<float> out({rows, cols});
+        std::copy(X.begin(), X.end(), out.mutable_data());
+        return out;
+    }, py::arg("rows"), py::arg("cols"), py::arg("seed") = 42, "Dense (rows, cols) float32 operand, uniform in [-1, 1)");
     mod.def("reload_tuning", []() { sparseops::check(so_tuning_reload(sparseops::context()), "so_tuning_reload"); },
             "Read the SPARSEOPS_* tuning overrides from the environment again (they are read when the process-wide "
             "context is created); models pick the change up at their next resize_buffers");

@@ -208,6 +208,16 @@ int main(int argc, char **argv)
         check(c.device.get() == state, "repeated conv2d_* calls reuse the layer's device state");
     }
 
+    {   // the reference's layer-chain types are declared with its names (include/sparse_onnx.hpp:30-138)
+        PoolAttr pool;
+        pool.kH = pool.kW = 3; pool.sH = pool.sW = 2; pool.C = 64;
+        Layer L{LayerType::Pool, LayerOp::MaxPool, LayerAttr{pool}, {"x"}, {"y"}};
+        RunResult rr{nullptr, 64u, false};
+        const DataLayout lay = DataLayout::PatchMajor;
+        check(std::get<PoolAttr>(L.attr).kH == 3 && L.inputs.size() == 1 && L.op == LayerOp::MaxPool && rr.features == 64u &&
+              !rr.owned && lay != DataLayout::NCHW_C, "Layer / LayerAttr / RunResult / DataLayout");
+    }
+
     if (argc == 5) {
         const uint32_t B = (uint32_t)std::atoi(argv[4]);
         const std::vector<float> in = read_floats(argv[2]), expected = read_floats(argv[3]);

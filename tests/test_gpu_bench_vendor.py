@@ -59,3 +59,15 @@ def test_vendor_runs_a_datagen_matrix(tmp_path):
     assert len(diffs) >= 4 and max(diffs) <= TOL, text
     text, diffs = run_vendor(["matvec", "--ellpack-file", path, "--runs", "3"])
     assert len(diffs) >= 4 and max(diffs) <= TOL, text
+
+
+@pytest.mark.parametrize("irregular", [0, 1])
+def test_vendor_and_python_draw_the_same_matrix(irregular):
+    """One generator (bench/data_gen.hpp) behind the harness and sparseops_backend.benchmark_dense:
+    the same seed gives the same matrix, so the harness's nnz and ELLPACK r are those of the Python side's."""
+    import sparseops_backend as sb
+    W = sb.benchmark_dense(384, 512, 0.9, 7, bool(irregular))
+    E = datagen.encode_dense(W)
+    text, _ = run_vendor(["matmul", "--M", "384", "--N", "512", "--C", "64", "--sparsity", "0.9", "--runs", "2",
+                          "--seed", "7", "--irregular", str(irregular)])
+    assert "nnz %d, ELLPACK r %d" % (np.count_nonzero(W), E.r) in text, text

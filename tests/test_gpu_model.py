@@ -329,7 +329,7 @@ def test_cpp_caller_of_the_reference_headers(oracle, tmp_path):
     r = subprocess.run([exe, path, str(tmp_path / "in.bin"), str(tmp_path / "expected.bin"), str(B)],
                        capture_output=True, text=True, timeout=100)
     assert r.returncode == 0, r.stdout + r.stderr
-    assert r.stdout.count("ok  ") == 18 and "FAIL" not in r.stdout
+    assert r.stdout.count("ok  ") == 19 and "FAIL" not in r.stdout
 
 
 def _run_device(model, ctx, X_bm):

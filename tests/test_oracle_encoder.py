@@ -132,3 +132,24 @@ def test_datagen_gap_generator_is_a_valid_encoding(oracle):
     Eo = oracle.encode(W)
     assert E.r == Eo.r and np.array_equal(E.Wd, Eo.Wd) and np.array_equal(E.idx, Eo.idx) and np.array_equal(E.nnz, Eo.nnz)
     assert abs(E.total_nnz / (300 * 2000) - 0.05) < 0.005
+
+
+def test_benchmark_generator(backend):
+    """sparseops_backend.benchmark_dense / benchmark_operand (bench/data_gen.hpp, the recipe of the reference's
+    benchmark-mkl/common/data_gen.cpp:23-96): deterministic per seed, a Bernoulli(1 - sparsity) mask over N(0,1)
+    values, a dense last row with `irregular`, operand uniform in [-1, 1)."""
+    W = backend.benchmark_dense(300, 400, 0.9, 11, False)
+    assert W.shape == (300, 400) and W.dtype == np.float32
+    assert np.array_equal(W, backend.benchmark_dense(300, 400, 0.9, 11, False))
+    assert not np.array_equal(W, backend.benchmark_dense(300, 400, 0.9, 12, False))
+    kept = np.count_nonzero(W) / W.size
+    assert abs(kept - 0.1) < 0.01
+    vals = W[W != 0]
+    assert abs(vals.mean()) < 0.05 and abs(vals.std() - 1.0) < 0.05
+    Wi = backend.benchmark_dense(50, 64, 0.9, 3, True)
+    assert np.count_nonzero(Wi[-1]) == 64 and np.count_nonzero(Wi[:-1]) < 0.2 * Wi[:-1].size
+    assert np.count_nonzero(backend.benchmark_dense(16, 16, 1.0, 1, False)) == 0
+    X = backend.benchmark_operand(128, 32, 5)
+    assert X.shape == (128, 32) and X.min() >= -1.0 and X.max() < 1.0 and abs(X.mean()) < 0.05
+    with pytest.raises(RuntimeError):
+        backend.benchmark_dense(4, 4, 1.5, 1, False)
