@@ -448,10 +448,11 @@ def main():
                      "t_hbm_us": round(nbytes / (HBM_PEAK_GBS * 1e9) * 1e6, 2),
                      "t_valu_us": round(flops / (VALU_FP32_PEAK_TF * 1e12) * 1e6, 2),
                      "t_bound_over_t": round(max(nbytes / (HBM_PEAK_GBS * 1e9), flops / (VALU_FP32_PEAK_TF * 1e12)) / (ev_ms * 1e-3), 4),
-                     "binding_bound": "not HBM (t_hbm 2.7 us): the multiply-adds themselves -- one register-indexed v_fmac_f32_dpp plus one "
-                                      "M0 write per nonzero and 64 columns, a dependent pair that takes a wave 10 clk: 3.4 clk per SIMD at the "
-                                      "kernel's 3 waves per SIMD, 10.7 us for the launch's 6.9 M pairs -- then waiting for the records' scalar "
-                                      "loads, the sums of the 12 x 2 partial tiles per output tile (LDS, then memory) and the launch's start-up"},
+                     "binding_bound": "not HBM (t_hbm 2.7 us).  From knock-out builds: 3.2 us launch and set-up; ~17 us the loop, bound twice "
+                                      "over -- a SIMD issues one scalar instruction per ~4 clk and every nonzero x 64 columns needs an M0 write "
+                                      "before its register-indexed v_fmac_f32_dpp (15.5 us with all loads removed), and every iteration of 64 pairs "
+                                      "waits one scalar-load round trip (16 us with the multiply-adds removed); 4.8 us the sum of a workgroup's 12 "
+                                      "partial tiles through LDS; 2.0 us the exchange of partial tiles between the two workgroups of an output tile"},
     }
     if args.calibrate_copy:
         # A plain copy of known size (act_kernel<NONE>: reads N floats, writes N floats)
