@@ -186,9 +186,10 @@ so_status so_ellpack_decode(so_ctx *ctx, const so_ellpack *E, float *dDense);
  * (include/ellpack_matmul.hpp:23-43).  dBias may be NULL (zero start). */
 so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
                     const float *dBias, float *dY, int act);
-/* Makes sure a later so_matmul(ctx, E, ..., C, ...) allocates nothing: on a handle with the RBM layout the
- * context's workspace is grown to what C dense columns need (a no-op for every other layout).  so_matmul
- * does this itself on first use of a larger output, but not while a graph is being recorded: a caller that
+/* Makes sure a later so_matmul(ctx, E, ..., C, ...) allocates and prepares nothing: on a handle with the RBM
+ * layout the context's workspace is grown to what C dense columns need and the handle's records are written
+ * for that width (a no-op for every other layout).  so_matmul does both itself on first use of a larger output
+ * or another width, but refuses to while a graph is being recorded: a caller that
  * records so_matmul into a graph calls this first (SparseOnnxModel::resize_buffers does, for every fully
  * connected layer -- the reference's documented way to get its allocation-free run(), README.md:146).
  * No counterpart in the reference. */

@@ -279,7 +279,8 @@ extern "C" so_status so_matmul_reserve(so_ctx *ctx, const so_ellpack *E, uint32_
 {
     SO_REQUIRE(ctx && E, "so_matmul_reserve: null argument");
     if (E->m == 0 || C == 0 || !so_matmul_rbm_applies(ctx, E, C)) return SO_OK;
-    return so_matmul_rbm_reserve(ctx, E, C);
+    const so_status st = so_matmul_rbm_reserve(ctx, E, C);
+    return st != SO_OK ? st : so_matmul_rbm_set_pitch(ctx, E, C);
 }
 
 extern "C" so_status so_matmul(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,

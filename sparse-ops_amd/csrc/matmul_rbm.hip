@@ -366,20 +366,29 @@ so_status so_matmul_rbm_reserve(so_ctx *ctx, const so_ellpack *E, uint32_t C)
     return SO_OK;
 }
 
+// The records address X rows by byte offset (row * pitch): rewritten for dense width C when the handle was
+// last used with another (stream-ordered; launches of one handle with different C must not overlap on
+// different streams).  Never inside a recording: the rewrite would become a node of the graph, run again
+// on every replay, and leave launches outside the graph with records that were never written.
+so_status so_matmul_rbm_set_pitch(so_ctx *ctx, const so_ellpack *E, uint32_t C)
+{
+    const so_rbmm &R = E->rbmm;
+    if (R.pitch == C * 4u) return SO_OK;
+    SO_REQUIRE(!ctx->capturing, "so_matmul: the row-block-merged records must be rewritten for %u dense columns, which cannot be done "
+                                "while a graph is being recorded (call so_matmul_reserve, or launch this shape once, before recording)", C);
+    so_rbmm &Rw = const_cast<so_ellpack *>(E)->rbmm;
+    const uint64_t words = R.nrec * 4;
+    rbmm_offsets_kernel<<<so_ceil_div(words, 256), 256, 0, ctx->stream>>>(Rw.d_rec, Rw.d_xrows, R.nrec, C * 4u);
+    Rw.pitch = C * 4u;
+    return SO_OK;
+}
+
 so_status so_matmul_rbm_launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
                                const float *dBias, float *dY, int act)
 {
-    const so_rbmm &R = E->rbmm;
-    const so_status rs = so_matmul_rbm_reserve(ctx, E, C);
+    so_status rs = so_matmul_rbm_reserve(ctx, E, C);
     if (rs != SO_OK) return rs;
-    if (R.pitch != C * 4u) {
-        // the handle's records are rewritten for this pitch (stream-ordered; launches of one handle with
-        // different C must not overlap on different streams)
-        so_rbmm &Rw = const_cast<so_ellpack *>(E)->rbmm;
-        const uint64_t words = R.nrec * 4;
-        rbmm_offsets_kernel<<<so_ceil_div(words, 256), 256, 0, ctx->stream>>>(Rw.d_rec, Rw.d_xrows, R.nrec, C * 4u);
-        Rw.pitch = C * 4u;
-    }
+    if ((rs = so_matmul_rbm_set_pitch(ctx, E, C)) != SO_OK) return rs;
     switch (act) {
     case SO_ACT_RELU:    return launch_rbm<SO_ACT_RELU>(ctx, E, dX, C, dBias, dY);
     case SO_ACT_SIGMOID: return launch_rbm<SO_ACT_SIGMOID>(ctx, E, dX, C, dBias, dY);

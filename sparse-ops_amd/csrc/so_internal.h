@@ -141,6 +141,7 @@ so_status so_matmul_tiled_launch(so_ctx *ctx, const so_ellpack *E, const float *
 so_status so_rbmm_build(so_ctx *ctx, so_ellpack *E, const float *Wd, const uint32_t *idx, const uint32_t *nnz);
 void so_rbmm_free(so_ellpack *E);
 bool so_matmul_rbm_applies(const so_ctx *ctx, const so_ellpack *E, uint32_t C);
+so_status so_matmul_rbm_set_pitch(so_ctx *ctx, const so_ellpack *E, uint32_t C);
 so_status so_matmul_rbm_reserve(so_ctx *ctx, const so_ellpack *E, uint32_t C);
 so_status so_matmul_rbm_launch(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C,
                                const float *dBias, float *dY, int act);

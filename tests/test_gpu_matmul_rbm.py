@@ -162,3 +162,50 @@ def test_rbm_default_dispatch_and_workspace_growth(ctx, oracle):
         for a in (dX, dY, dB):
             a.free()
     dE.free()
+
+
+def test_rbm_in_a_launch_graph(ctx, oracle):
+    """so_matmul_reserve sizes the workspace ahead of time, so that a launch of the kernel whose workgroups
+    exchange partial tiles (ksplit 2) can be recorded; the graph replays with the eager launch's bits, several
+    times, with eager launches of the same handle and synchronisation in between.  Recording without the
+    reservation is refused (the workspace cannot grow inside a recording), and the refusal leaves the context usable."""
+    rng = np.random.default_rng(17)
+    W = sparse_matrix(rng, 512, 1600, .9)
+    E = datagen.encode_dense(W)
+    b = rng.standard_normal(512).astype(np.float32)
+    C = 128
+    with ctx.tuning(SPARSEOPS_MATMUL_RBM="1", SPARSEOPS_MATMUL_RBM_SPLIT="2"):
+        fresh = hipabi.Context(0)                      # a context whose workspace is still empty
+        try:
+            fE = fresh.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, RBM)
+            fX, fY = fresh.empty((1600, C)), fresh.empty((512, C))
+            fresh.graph_begin()
+            with pytest.raises(hipabi.SoError, match="so_matmul_reserve"):
+                fresh.matmul(fE, fX, C, None, fY, "none")
+            g0 = fresh.graph_end()
+            fresh.graph_free(g0)
+            fresh.matmul(fE, fX, C, None, fY, "none")   # eager launches still work
+            fresh.sync()
+        finally:
+            fresh.close()
+        dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, RBM)
+        dX, dY, dB = ctx.empty((1600, C)), ctx.empty((512, C)), ctx.array(b)
+        ctx.matmul_reserve(dE, C)
+        ctx.graph_begin()
+        ctx.matmul(dE, dX, C, dB, dY, "relu")
+        g = ctx.graph_end()
+        for it in range(4):
+            X = rng.standard_normal((1600, C)).astype(np.float32)
+            dX.upload(X)
+            ctx.matmul(dE, dX, C, dB, dY, "relu")
+            eager = dY.download()
+            ctx.fill_zero(dY)
+            ctx.sync()
+            ctx.graph_launch(g)
+            Y = dY.download()
+            assert np.array_equal(Y, eager), it
+            assert rel_err(Y, oracle.matmul(as_oracle(E), X, b, "relu")) <= TOL
+        ctx.graph_free(g)
+        for a in (dX, dY, dB):
+            a.free()
+        dE.free()

@@ -402,3 +402,37 @@ def test_model_runs_the_row_block_merged_plan(backend, oracle, tmp_path, B):
         backend.reload_tuning()
     assert np.array_equal(outs["1"], outs["0"]) and np.array_equal(outs[None], outs["0"])
     assert np.array_equal(outs["0"][:2], run_graph(oracle, payload, X[:2]))
+
+
+def test_deep_mlp_records_the_row_block_merged_kernel(backend, oracle, tmp_path):
+    """Nine 1024-wide layers at batch 256: a chain long enough to be recorded into a launch graph, whose large
+    layers run on the row-block-merged matmul (workspace and records prepared by resize_buffers, outside the
+    recording).  Replays, an eager model (SPARSEOPS_NO_GRAPH=1) and a second batch size agree bit for bit with
+    one another; against the in-order CPU chain the result is within the tolerance of that kernel."""
+    rng = np.random.default_rng(91)
+    Ws = [datagen.magnitude_prune((rng.standard_normal((1024, 1024)) * 0.08).astype(np.float32), .9) for _ in range(9)]
+    acts = ["Relu"] * 8 + [None]
+    path = ow.save(str(tmp_path / "deep.onnx"), ow.mlp_model(Ws, acts, 256))
+    X = rng.standard_normal((256, 1024)).astype(np.float32)
+    Yo = oracle_mlp(oracle, Ws, acts, X)
+    outs = {}
+    os.environ["SPARSEOPS_MATMUL_RBM"] = "1"                   # 1024-row layers do not cover the chip: ask for the kernel
+    try:
+        for no_graph in ("0", "1"):
+            os.environ["SPARSEOPS_NO_GRAPH"] = no_graph
+            backend.reload_tuning()
+            model = backend.SparseOnnxModel(path)
+            outs[no_graph] = [model.run(X) for _ in range(3)]
+            if no_graph == "0":
+                model.resize_buffers(128)                      # other width: records rewritten, graph re-recorded
+                half = [model.run(X[:128]) for _ in range(2)]
+                model.resize_buffers(256)
+                outs["back"] = [model.run(X)]
+    finally:
+        del os.environ["SPARSEOPS_NO_GRAPH"], os.environ["SPARSEOPS_MATMUL_RBM"]
+        backend.reload_tuning()
+    assert not np.array_equal(outs["0"][0], Yo)                # the in-order kernels would give the CPU chain's bits
+    for Y in outs["0"] + outs["1"] + outs["back"]:
+        assert np.array_equal(Y, outs["0"][0])
+    assert np.array_equal(half[0], half[1])
+    assert rel_err(outs["0"][0], Yo) <= 1e-4 and rel_err(half[0], Yo[:128]) <= 1e-4
