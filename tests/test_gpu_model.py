@@ -405,18 +405,18 @@ def test_model_runs_the_row_block_merged_plan(backend, oracle, tmp_path, B):
 
 
 def test_deep_mlp_records_the_row_block_merged_kernel(backend, oracle, tmp_path):
-    """Nine 1024-wide layers at batch 256: a chain long enough to be recorded into a launch graph, whose large
+    """Nine 1536-wide layers at batch 256: a chain long enough to be recorded into a launch graph, whose large
     layers run on the row-block-merged matmul (workspace and records prepared by resize_buffers, outside the
     recording).  Replays, an eager model (SPARSEOPS_NO_GRAPH=1) and a second batch size agree bit for bit with
     one another; against the in-order CPU chain the result is within the tolerance of that kernel."""
     rng = np.random.default_rng(91)
-    Ws = [datagen.magnitude_prune((rng.standard_normal((1024, 1024)) * 0.08).astype(np.float32), .9) for _ in range(9)]
+    Ws = [datagen.magnitude_prune((rng.standard_normal((1536, 1536)) * 0.07).astype(np.float32), .9) for _ in range(9)]
     acts = ["Relu"] * 8 + [None]
     path = ow.save(str(tmp_path / "deep.onnx"), ow.mlp_model(Ws, acts, 256))
-    X = rng.standard_normal((256, 1024)).astype(np.float32)
+    X = rng.standard_normal((256, 1536)).astype(np.float32)
     Yo = oracle_mlp(oracle, Ws, acts, X)
     outs = {}
-    os.environ["SPARSEOPS_MATMUL_RBM"] = "1"                   # 1024-row layers do not cover the chip: ask for the kernel
+    os.environ["SPARSEOPS_MATMUL_RBM"] = "1"                   # 1536-row layers do not cover the chip: ask for the kernel
     try:
         for no_graph in ("0", "1"):
             os.environ["SPARSEOPS_NO_GRAPH"] = no_graph
