@@ -209,3 +209,37 @@ def test_rbm_in_a_launch_graph(ctx, oracle):
         for a in (dX, dY, dB):
             a.free()
         dE.free()
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_rbm_random_sweep(ctx, oracle, seed):
+    """Seeded random shapes, densities, K splits and sparsity patterns (uniform, a few dense columns, a few dense
+    rows, whole empty row blocks) against the oracle and the fp64 product."""
+    rng = np.random.default_rng(1000 + seed)
+    m = int(rng.integers(1, 700))
+    n = int(rng.integers(1, 2500))
+    C = int(rng.choice([1, 3, 17, 63, 64, 65, 128, 200, 256, 333]))
+    density = float(rng.choice([0.01, 0.05, 0.1, 0.3, 0.7]))
+    W = (rng.standard_normal((m, n)) * (rng.random((m, n)) < density)).astype(np.float32)
+    pattern = seed % 4
+    if pattern == 1:                                   # columns that every row uses: parts of 16 pairs, many per column
+        cols = rng.choice(n, size=min(n, 3), replace=False)
+        W[:, cols] = rng.standard_normal((m, len(cols))).astype(np.float32)
+    elif pattern == 2:                                 # dense rows: r = n
+        rows = rng.choice(m, size=min(m, 2), replace=False)
+        W[rows, :] = rng.standard_normal((len(rows), n)).astype(np.float32)
+    elif pattern == 3 and m > 128:                     # a whole 128-row block without nonzeros
+        W[:128, :] = 0
+    X = rng.standard_normal((n, C)).astype(np.float32)
+    b = rng.standard_normal(m).astype(np.float32) if seed % 3 else None
+    E = datagen.encode_dense(W)
+    split = [None, 1, 2, 4][int(rng.integers(0, 4))]
+    act = ["none", "relu"][seed % 2]
+    Y = rbm_matmul(ctx, E, X, b, act=act, split=split, repeat=2)
+    Yo = oracle.matmul(as_oracle(E), X, b, act)
+    assert Y.shape == Yo.shape
+    ref64 = W.astype(np.float64) @ X.astype(np.float64) + (0 if b is None else b[:, None].astype(np.float64))
+    if act == "relu":
+        ref64 = np.maximum(ref64, 0)
+    scale = max(np.abs(ref64).max(), 1e-30)
+    assert np.abs(Y - Yo).max() <= TOL * scale and np.abs(Y - ref64).max() <= TOL * scale
