@@ -43,8 +43,8 @@ LDS_OPERAND_PEAK_TF = 78.6   # 256 CUs x 256 B/clk of ds_read_b128 (measured 255
 TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 HEADLINE_KERNEL = "ellpack_matmul_rbm_kernel<0>"
 TILED_KERNEL = "ellpack_matmul_tiled_kernel<0>"
-MATVEC_KERNELS = {"ellpack_matvec 16384x16384, 95% Bernoulli": ("matvec_rows_kernel", "matvec 16384^2 uniform"),
-                  "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048": ("matvec_binned_kernel", "matvec 16384^2 zipf")}
+MATVEC_KERNELS = {"ellpack_matvec 16384x16384, 95% Bernoulli": ("matvec_rows_kernel<true,64,true>", "matvec 16384^2 uniform"),
+                  "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048": ("matvec_binned_kernel<true,true>", "matvec 16384^2 zipf")}
 
 
 def measured_traffic(kernel, workload=None):
@@ -220,17 +220,28 @@ def cpu_baseline_matvec(E, x, b, y_gpu, nbytes):
 
 def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup, with_cpu=True):
     E, x, b = gen()
+    # Up to 65536 columns the handle also keeps them in 16 bits (SO_LAYOUT_IDX16) and so_matvec streams 6 bytes
+    # per nonzero instead of the format's 8: same bits, a quarter less to read.  `alg_bytes` and `hbm_frac` stay
+    # on the reference format's 8 bytes per nonzero; `bytes_read` / `hbm_frac_bytes_read` are what the kernel
+    # actually streams, and `idx32` is the same handle with the 32-bit columns.
+    compact = E.n <= 65536
+    if compact:
+        layouts |= hipabi.LAYOUT_IDX16
     dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, layouts)
     dx, dB, dy = ctx.array(x), ctx.array(b), ctx.empty((E.m,))
     _, ms = time_launches(ctx, lambda: ctx.matvec(dE, dx, dB, dy, layout), steps, warmup)
-    nbytes = 8 * E.total_nnz + 4 * E.m + 4 * E.m + 4 * E.n + 4 * E.m
+    vectors = 4 * E.m + 4 * E.m + 4 * E.n + 4 * E.m
+    nbytes = 8 * E.total_nnz + vectors
+    nread = (6 if compact else 8) * E.total_nnz + vectors
     out = {"workload": name, "m": E.m, "n": E.n, "r": E.r, "nnz": E.total_nnz, "us_per_launch": round(ms * 1e3, 2),
            "alg_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1), "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+           "column_bits": 16 if compact else 32, "bytes_read": nread,
+           "hbm_frac_bytes_read": round(nread / ms / 1e6 / HBM_PEAK_GBS, 4),
            "padded_bytes": 8 * E.m * E.r,
            "traffic": measured_traffic(*MATVEC_KERNELS[name]) if name in MATVEC_KERNELS else None}
     if with_cpu:
         out["cpu_baseline"] = cpu_baseline_matvec(E, x, b, dy.download(), nbytes)
-    # Cache-cold figure: the streamed arrays (66-108 MB) fit the 256 MB Infinity Cache when the
+    # Cache-cold figure: the streamed arrays (50-108 MB) fit the 256 MB Infinity Cache when the
     # same launch repeats back to back, so also rotate the launches over enough copies of the
     # matrix that a copy has been evicted by the time its turn comes again.
     copies = [dE] + [ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, layouts) for _ in range(5)]
@@ -239,10 +250,22 @@ def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup
     def rotate():
         ctx.matvec(copies[turn[0] % len(copies)], dx, dB, dy, layout)
         turn[0] += 1
-    _, cold_ms = time_launches(ctx, rotate, len(copies) * max(2, steps // len(copies)), len(copies))
+    cold_steps = len(copies) * max(2, steps // len(copies))
+    _, cold_ms = time_launches(ctx, rotate, cold_steps, len(copies))
     out["us_per_launch_cache_cold"] = round(cold_ms * 1e3, 2)
     out["hbm_frac_cache_cold"] = round(nbytes / cold_ms / 1e6 / HBM_PEAK_GBS, 4)
+    out["hbm_frac_bytes_read_cache_cold"] = round(nread / cold_ms / 1e6 / HBM_PEAK_GBS, 4)
     out["cache_cold_copies"] = len(copies)
+    if compact:
+        y16 = dy.download()
+        with ctx.tuning(SPARSEOPS_MATVEC_IDX16="0"):
+            _, ms32 = time_launches(ctx, lambda: ctx.matvec(dE, dx, dB, dy, layout), steps, warmup)
+            _, cold32 = time_launches(ctx, rotate, cold_steps, len(copies))
+            ctx.matvec(dE, dx, dB, dy, layout)
+        out["idx32"] = {"us_per_launch": round(ms32 * 1e3, 2), "hbm_frac": round(nbytes / ms32 / 1e6 / HBM_PEAK_GBS, 4),
+                        "us_per_launch_cache_cold": round(cold32 * 1e3, 2),
+                        "hbm_frac_cache_cold": round(nbytes / cold32 / 1e6 / HBM_PEAK_GBS, 4),
+                        "same_bits_as_16_bit_columns": bool(np.array_equal(y16, dy.download()))}
     for c in copies[1:]:
         c.free()
     dE.free()

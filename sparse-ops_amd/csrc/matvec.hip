@@ -5,7 +5,8 @@
 // bandwidth: x is staged once per workgroup in LDS when it fits (the gathers
 // then never leave the CU), the pairs are read with 16-byte non-temporal loads,
 // four per lane in flight, and only the first nnz[i] slots of a row are touched,
-// so ELLPACK padding is never streamed.
+// so ELLPACK padding is never streamed.  A handle uploaded with SO_LAYOUT_IDX16 also has
+// its columns in 16 bits: the row-major kernels then stream 6 bytes per nonzero.
 //
 //   rows kernel    one wavefront per row on the row-major arrays; lanes take
 //                  aligned groups of four slots, partial sums are combined with a
@@ -30,6 +31,26 @@ constexpr int kWavesPerBlock = kBlock / 64;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// The columns of four consecutive slots as they are loaded: four 32-bit words, or two when the
+// handle carries its columns in 16 bits as well (SO_LAYOUT_IDX16: 6 bytes per nonzero instead of 8).
+template <bool I16> struct ColGroup;
+template <> struct ColGroup<false> {
+    using T = u32x4;
+    using E = uint32_t;
+    static __device__ __forceinline__ u32x4 cols(T t) { return t; }
+};
+template <> struct ColGroup<true> {
+    using T = u32x2;
+    using E = uint16_t;
+    static __device__ __forceinline__ u32x4 cols(T t)
+    {
+        u32x4 c;
+        c.x = t.x & 0xffffu; c.y = t.x >> 16; c.z = t.y & 0xffffu; c.w = t.y >> 16;
+        return c;
+    }
+};
 
 template <int G>
 __device__ __forceinline__ float group_sum(float v)
@@ -57,15 +78,16 @@ __device__ __forceinline__ const float *stage_x(const float *__restrict__ x, uin
 // them.  The row's slots [beg, end) are covered by aligned groups of four; a lane loads up to four
 // such groups (addresses past the row are clamped onto its last group and every slot outside
 // [beg, end) is masked to an exact no-op).  Rows longer than 1024 slots continue in row_rest.
+template <bool I16>
 struct RowLoads {
     f32x4 w[4];
-    u32x4 c[4];
+    typename ColGroup<I16>::T c[4];
 };
 
 // G = lanes that share a row (64, 32, 16 or 8): a pass of the row covers 16 G slots.
-template <int G = 64>
-__device__ __forceinline__ void row_issue(const f32x4 *__restrict__ Wd4, const u32x4 *__restrict__ idx4,
-                                          uint64_t beg, uint64_t end, uint64_t q0, RowLoads &L)
+template <int G, bool I16>
+__device__ __forceinline__ void row_issue(const f32x4 *__restrict__ Wd4, const typename ColGroup<I16>::T *__restrict__ idx4,
+                                          uint64_t beg, uint64_t end, uint64_t q0, RowLoads<I16> &L)
 {
     const uint64_t qlast = end > beg ? (end - 1) >> 2 : beg >> 2;
 #pragma unroll
@@ -76,8 +98,8 @@ __device__ __forceinline__ void row_issue(const f32x4 *__restrict__ Wd4, const u
     }
 }
 
-template <int G = 64>
-__device__ __forceinline__ void row_consume(const RowLoads &L, uint64_t beg, uint64_t end, uint64_t q0, const float *xs,
+template <int G, bool I16>
+__device__ __forceinline__ void row_consume(const RowLoads<I16> &L, uint64_t beg, uint64_t end, uint64_t q0, const float *xs,
                                             float &a0, float &a1, float &a2, float &a3)
 {
     // slot k of group u is live iff its distance from the row's start is in [0, end - beg): one
@@ -89,8 +111,9 @@ __device__ __forceinline__ void row_consume(const RowLoads &L, uint64_t beg, uin
         const int32_t rel = rel0 + 4 * G * u;
         const bool v0 = (uint32_t)rel < len, v1 = (uint32_t)(rel + 1) < len;
         const bool v2 = (uint32_t)(rel + 2) < len, v3 = (uint32_t)(rel + 3) < len;
-        const float x0 = xs[v0 ? L.c[u].x : 0u], x1 = xs[v1 ? L.c[u].y : 0u];
-        const float x2 = xs[v2 ? L.c[u].z : 0u], x3 = xs[v3 ? L.c[u].w : 0u];
+        const u32x4 c = ColGroup<I16>::cols(L.c[u]);
+        const float x0 = xs[v0 ? c.x : 0u], x1 = xs[v1 ? c.y : 0u];
+        const float x2 = xs[v2 ? c.z : 0u], x3 = xs[v3 ? c.w : 0u];
         a0 = __builtin_fmaf(v0 ? L.w[u].x : 0.0f, v0 ? x0 : 0.0f, a0);
         a1 = __builtin_fmaf(v1 ? L.w[u].y : 0.0f, v1 ? x1 : 0.0f, a1);
         a2 = __builtin_fmaf(v2 ? L.w[u].z : 0.0f, v2 ? x2 : 0.0f, a2);
@@ -99,22 +122,23 @@ __device__ __forceinline__ void row_consume(const RowLoads &L, uint64_t beg, uin
 }
 
 // The whole row at once (used where rows are not pipelined).
-__device__ __forceinline__ float wave_row_dot(const f32x4 *__restrict__ Wd4, const u32x4 *__restrict__ idx4,
+template <bool I16>
+__device__ __forceinline__ float wave_row_dot(const f32x4 *__restrict__ Wd4, const typename ColGroup<I16>::T *__restrict__ idx4,
                                               uint64_t beg, uint64_t end, const float *xs, uint32_t lane)
 {
     float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
     if (end == beg) return 0.0f;
     const uint64_t qlast = (end - 1) >> 2;
     for (uint64_t q0 = (beg >> 2) + lane; q0 <= qlast; q0 += 256) {
-        RowLoads L;
-        row_issue(Wd4, idx4, beg, end, q0, L);
-        row_consume(L, beg, end, q0, xs, a0, a1, a2, a3);
+        RowLoads<I16> L;
+        row_issue<64, I16>(Wd4, idx4, beg, end, q0, L);
+        row_consume<64, I16>(L, beg, end, q0, xs, a0, a1, a2, a3);
     }
     return group_sum<64>((a0 + a1) + (a2 + a3));
 }
 
-template <int G>
-__device__ __forceinline__ float group_row_dot(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
+template <int G, typename IdxT>
+__device__ __forceinline__ float group_row_dot(const float *__restrict__ Wd, const IdxT *__restrict__ idx,
                                                uint64_t base, uint32_t cnt, const float *xs, uint32_t sub)
 {
     float a = 0.0f;
@@ -124,9 +148,9 @@ __device__ __forceinline__ float group_row_dot(const float *__restrict__ Wd, con
 
 // G lanes per row: a wave works on 64/G rows at a time (whole waves for rows longer than 512
 // slots, a half, a quarter or an eighth of a wave for shorter ones, so that short rows do not leave lanes idle).
-template <bool XLDS, int G>
+template <bool XLDS, int G, bool I16>
 __global__ __launch_bounds__(kBlock)
-void matvec_rows_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
+void matvec_rows_kernel(const float *__restrict__ Wd, const void *__restrict__ idx,
                         const uint32_t *__restrict__ nnz, uint32_t count, uint32_t r,
                         const float *__restrict__ x, uint32_t n,
                         const float *__restrict__ bias, float *__restrict__ y)
@@ -137,7 +161,7 @@ void matvec_rows_kernel(const float *__restrict__ Wd, const uint32_t *__restrict
     const uint32_t wave = __builtin_amdgcn_readfirstlane(blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6));
     const uint32_t stride = gridDim.x * kWavesPerBlock * RPW;            // rows between a group's consecutive rows
     const f32x4 *Wd4 = reinterpret_cast<const f32x4 *>(Wd);
-    const u32x4 *idx4 = reinterpret_cast<const u32x4 *>(idx);
+    const typename ColGroup<I16>::T *idx4 = reinterpret_cast<const typename ColGroup<I16>::T *>(idx);
     // Rows are pipelined: the first 16 G slots of the next row are requested before the current
     // row is reduced, and those of the group's first row before x is staged, so that a wave always
     // has a row's worth of loads in flight.  Row lengths are fetched two rows ahead, so that
@@ -145,24 +169,24 @@ void matvec_rows_kernel(const float *__restrict__ Wd, const uint32_t *__restrict
     uint32_t row = wave * RPW + grp;
     uint64_t beg = (uint64_t)row * r, end = beg + (row < count ? nnz[row] : 0u);
     uint32_t len1 = (uint64_t)row + stride < count ? nnz[row + stride] : 0u;          // length of the next row
-    RowLoads cur, nxt;
-    if (row < count) row_issue<G>(Wd4, idx4, beg, end, (beg >> 2) + sub, cur);
+    RowLoads<I16> cur, nxt;
+    if (row < count) row_issue<G, I16>(Wd4, idx4, beg, end, (beg >> 2) + sub, cur);
     const float *xs = stage_x<XLDS>(x, n, lds_x);
     // all groups of a wave make the same number of trips (the reductions need every lane)
     for (uint32_t base = wave * RPW; base < count; base += stride, row += stride) {
         const uint64_t nrow = (uint64_t)row + stride;
         const uint64_t nbeg = nrow * r, nend = nbeg + len1;
-        if (nrow < count) row_issue<G>(Wd4, idx4, nbeg, nend, (nbeg >> 2) + sub, nxt);
+        if (nrow < count) row_issue<G, I16>(Wd4, idx4, nbeg, nend, (nbeg >> 2) + sub, nxt);
         const uint32_t len2 = nrow + stride < count ? nnz[nrow + stride] : 0u;
         float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
         if (row < count && end > beg) {
             const uint64_t qlast = (end - 1) >> 2;
             uint64_t q0 = (beg >> 2) + sub;
-            row_consume<G>(cur, beg, end, q0, xs, a0, a1, a2, a3);
+            row_consume<G, I16>(cur, beg, end, q0, xs, a0, a1, a2, a3);
             for (q0 += 4 * G; q0 <= qlast; q0 += 4 * G) {        // rows longer than one pass
-                RowLoads more;
-                row_issue<G>(Wd4, idx4, beg, end, q0, more);
-                row_consume<G>(more, beg, end, q0, xs, a0, a1, a2, a3);
+                RowLoads<I16> more;
+                row_issue<G, I16>(Wd4, idx4, beg, end, q0, more);
+                row_consume<G, I16>(more, beg, end, q0, xs, a0, a1, a2, a3);
             }
         }
         const float s = group_sum<G>((a0 + a1) + (a2 + a3));
@@ -176,8 +200,8 @@ void matvec_rows_kernel(const float *__restrict__ Wd, const uint32_t *__restrict
 
 // Rows of at most G*T nonzeros, G lanes per row.  Such a row is a chain of memory round trips and
 // nothing else, so all of a group's first row is requested before x is staged.
-template <bool XLDS, int G, int T>
-__device__ __forceinline__ void short_rows(const float *__restrict__ Wd, const uint32_t *__restrict__ idx,
+template <bool XLDS, int G, int T, typename IdxT>
+__device__ __forceinline__ void short_rows(const float *__restrict__ Wd, const IdxT *__restrict__ idx,
                                            const uint2 *__restrict__ rows, uint32_t count, uint32_t block, uint32_t blocks,
                                            uint32_t r, const float *__restrict__ x, uint32_t n, float *lds_x,
                                            const float *__restrict__ bias, float *__restrict__ y)
@@ -220,9 +244,9 @@ struct BinArgs {
     uint32_t b64, b16;                         // workgroups given to the 64- and 16-lane classes
 };
 
-template <bool XLDS>
+template <bool XLDS, bool I16>
 __global__ __launch_bounds__(kBlock, 8)          // 64 registers: two workgroups per compute unit
-void matvec_binned_kernel(const float *__restrict__ Wd, const uint32_t *__restrict__ idx, BinArgs ba, uint32_t r,
+void matvec_binned_kernel(const float *__restrict__ Wd, const void *__restrict__ idxv, BinArgs ba, uint32_t r,
                           const float *__restrict__ x, uint32_t n,
                           const float *__restrict__ bias, float *__restrict__ y)
 {
@@ -236,23 +260,23 @@ void matvec_binned_kernel(const float *__restrict__ Wd, const uint32_t *__restri
         const uint32_t lane = threadIdx.x & 63u;
         const uint32_t stride = ba.b64 * kWavesPerBlock;
         const f32x4 *Wd4 = reinterpret_cast<const f32x4 *>(Wd);
-        const u32x4 *idx4 = reinterpret_cast<const u32x4 *>(idx);
+        const typename ColGroup<I16>::T *idx4 = reinterpret_cast<const typename ColGroup<I16>::T *>(idxv);
         uint32_t g = __builtin_amdgcn_readfirstlane(b * kWavesPerBlock + (threadIdx.x >> 6));
         const uint2 e = g < ba.n64 ? ba.rows64[g] : make_uint2(0u, 0u);
         const uint64_t beg = (uint64_t)e.x * r, end = beg + e.y;
         const uint64_t q0 = (beg >> 2) + lane;
         const float *xs = stage_x<XLDS>(x, n, lds_x);
-        RowLoads A;
-        if (e.y > 0) row_issue(Wd4, idx4, beg, end, q0, A);
+        RowLoads<I16> A;
+        if (e.y > 0) row_issue<64, I16>(Wd4, idx4, beg, end, q0, A);
         if (g < ba.n64) {
             float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
             if (e.y > 0) {
-                row_consume(A, beg, end, q0, xs, a0, a1, a2, a3);
+                row_consume<64, I16>(A, beg, end, q0, xs, a0, a1, a2, a3);
                 const uint64_t qlast = (end - 1) >> 2;
                 for (uint64_t q = q0 + 256; q <= qlast; q += 256) {
-                    RowLoads L;
-                    row_issue(Wd4, idx4, beg, end, q, L);
-                    row_consume(L, beg, end, q, xs, a0, a1, a2, a3);
+                    RowLoads<I16> L;
+                    row_issue<64, I16>(Wd4, idx4, beg, end, q, L);
+                    row_consume<64, I16>(L, beg, end, q, xs, a0, a1, a2, a3);
                 }
             }
             const float s = group_sum<64>((a0 + a1) + (a2 + a3));
@@ -261,12 +285,14 @@ void matvec_binned_kernel(const float *__restrict__ Wd, const uint32_t *__restri
         for (g += stride; g < ba.n64; g += stride) {
             const uint2 en = ba.rows64[g];
             const uint64_t nbeg = (uint64_t)en.x * r;
-            const float s = wave_row_dot(Wd4, idx4, nbeg, nbeg + en.y, xs, lane);
+            const float s = wave_row_dot<I16>(Wd4, idx4, nbeg, nbeg + en.y, xs, lane);
             if (lane == 0) y[en.x] = (bias ? bias[en.x] : 0.0f) + s;
         }
     } else if (b < ba.b64 + ba.b16) {
+        const typename ColGroup<I16>::E *idx = reinterpret_cast<const typename ColGroup<I16>::E *>(idxv);
         short_rows<XLDS, 16, 8>(Wd, idx, ba.rows16, ba.n16, b - ba.b64, ba.b16, r, x, n, lds_x, bias, y);
     } else {
+        const typename ColGroup<I16>::E *idx = reinterpret_cast<const typename ColGroup<I16>::E *>(idxv);
         short_rows<XLDS, 4, 4>(Wd, idx, ba.rows4, ba.n4, b - ba.b64 - ba.b16, gridDim.x - ba.b64 - ba.b16, r, x, n,
                                lds_x, bias, y);
     }
@@ -325,6 +351,9 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
 
     const uint32_t cus = (uint32_t)ctx->compute_units;
     const size_t lds = (size_t)E->n * sizeof(float);
+    // the row-major kernels read the 16-bit copy of the columns when the handle has one
+    const bool i16 = E->d_idx16 != nullptr && ctx->tune.matvec_idx16 != 0;
+    const void *cols = i16 ? (const void *)E->d_idx16 : (const void *)E->d_idx;
     if (layout == SO_LAYOUT_ROW) {
         // Lanes per row by the longest row (one pass of 16 G slots should cover it), but never so
         // few that compute units are left without rows.
@@ -335,19 +364,25 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
         // One resident workgroup per compute unit (the pipelined rows need the registers); each of
         // its 16 waves keeps two passes' loads in flight.
         const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, kWavesPerBlock * (64u / G)), cus));
-#define SO_MV_ROWS(G)                                                                                              \
+#define SO_MV_ROWS(G, I16)                                                                                         \
         do {                                                                                                       \
-            if (use_lds(ctx, matvec_rows_kernel<true, G>, E->n, E->total_nnz, blocks))                             \
-                matvec_rows_kernel<true, G><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->r, \
-                                                                                  dx, E->n, dBias, dy);            \
+            if (use_lds(ctx, matvec_rows_kernel<true, G, I16>, E->n, E->total_nnz, blocks))                        \
+                matvec_rows_kernel<true, G, I16><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, cols, E->d_nnz, E->m, E->r, \
+                                                                                       dx, E->n, dBias, dy);       \
             else                                                                                                   \
-                matvec_rows_kernel<false, G><<<blocks, kBlock, 0, ctx->stream>>>(E->d_Wd, E->d_idx, E->d_nnz, E->m, E->r,  \
-                                                                                 dx, E->n, dBias, dy);             \
+                matvec_rows_kernel<false, G, I16><<<blocks, kBlock, 0, ctx->stream>>>(E->d_Wd, cols, E->d_nnz, E->m, E->r,  \
+                                                                                      dx, E->n, dBias, dy);        \
         } while (0)
-        if (G == 8) SO_MV_ROWS(8);
-        else if (G == 16) SO_MV_ROWS(16);
-        else if (G == 32) SO_MV_ROWS(32);
-        else SO_MV_ROWS(64);
+#define SO_MV_ROWS_G(I16)                                                                                          \
+        do {                                                                                                       \
+            if (G == 8) SO_MV_ROWS(8, I16);                                                                        \
+            else if (G == 16) SO_MV_ROWS(16, I16);                                                                 \
+            else if (G == 32) SO_MV_ROWS(32, I16);                                                                 \
+            else SO_MV_ROWS(64, I16);                                                                              \
+        } while (0)
+        if (i16) SO_MV_ROWS_G(true);
+        else SO_MV_ROWS_G(false);
+#undef SO_MV_ROWS_G
 #undef SO_MV_ROWS
     } else if (layout == SO_LAYOUT_SLOT) {
         const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, kBlock), 2u * cus));
@@ -368,12 +403,18 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
         const uint32_t b4 = std::min(so_ceil_div(ba.n4, kBlock / 4), std::max(1u, cus / 4));
         const uint32_t blocks = ba.b64 + ba.b16 + b4;
         if (blocks == 0) return SO_OK;
-        if (use_lds(ctx, matvec_binned_kernel<true>, E->n, E->total_nnz, blocks))
-            matvec_binned_kernel<true><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, E->d_idx, ba, E->r,
-                                                                             dx, E->n, dBias, dy);
-        else
-            matvec_binned_kernel<false><<<blocks, kBlock, 0, ctx->stream>>>(E->d_Wd, E->d_idx, ba, E->r,
-                                                                            dx, E->n, dBias, dy);
+#define SO_MV_BINNED(I16)                                                                                          \
+        do {                                                                                                       \
+            if (use_lds(ctx, matvec_binned_kernel<true, I16>, E->n, E->total_nnz, blocks))                         \
+                matvec_binned_kernel<true, I16><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, cols, ba, E->r,     \
+                                                                                      dx, E->n, dBias, dy);        \
+            else                                                                                                   \
+                matvec_binned_kernel<false, I16><<<blocks, kBlock, 0, ctx->stream>>>(E->d_Wd, cols, ba, E->r,      \
+                                                                                     dx, E->n, dBias, dy);         \
+        } while (0)
+        if (i16) SO_MV_BINNED(true);
+        else SO_MV_BINNED(false);
+#undef SO_MV_BINNED
     }
     SO_LAUNCH_CHECK();
     return SO_OK;

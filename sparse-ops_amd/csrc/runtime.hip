@@ -68,6 +68,7 @@ static void read_tuning(so_tuning &t)
     t.matmul_rbm_split = env_int("SPARSEOPS_MATMUL_RBM_SPLIT", 0);
     const int lanes = env_int("SPARSEOPS_MATVEC_LANES", 0);
     t.matvec_lanes = (lanes == 8 || lanes == 16 || lanes == 32 || lanes == 64) ? lanes : 0;
+    t.matvec_idx16 = env_int("SPARSEOPS_MATVEC_IDX16", -1);
     t.conv_min_cg = env_int("SPARSEOPS_CONV_MIN_CG", 0);
     t.conv_window = env_int("SPARSEOPS_CONV_WINDOW", -1);
     t.conv_cpw = env_int("SPARSEOPS_CONV_CPW", 0);
@@ -332,6 +333,7 @@ static void free_ellpack_arrays(so_ellpack *E)
     if (E->d_nnz) (void)hipFree(E->d_nnz);
     if (E->d_WdT) (void)hipFree(E->d_WdT);
     if (E->d_idxT) (void)hipFree(E->d_idxT);
+    if (E->d_idx16) (void)hipFree(E->d_idx16);
     for (auto &b : E->bins)
         if (b.d_rows) (void)hipFree(b.d_rows);
     if (E->tiled.d_entries) (void)hipFree(E->tiled.d_entries);
@@ -456,8 +458,9 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
     const size_t slots = (size_t)m * r;
     SO_REQUIRE(m == 0 || nnz != nullptr, "so_ellpack_upload: nnz is null");
     SO_REQUIRE(slots == 0 || (Wd && idx), "so_ellpack_upload: Wd/idx is null");
-    SO_REQUIRE((layouts & ~(SO_LAYOUT_ROW | SO_LAYOUT_SLOT | SO_LAYOUT_BINS | SO_LAYOUT_TILED | SO_LAYOUT_RBM)) == 0,
+    SO_REQUIRE((layouts & ~(SO_LAYOUT_ROW | SO_LAYOUT_SLOT | SO_LAYOUT_BINS | SO_LAYOUT_TILED | SO_LAYOUT_RBM | SO_LAYOUT_IDX16)) == 0,
                "so_ellpack_upload: unknown layout bits 0x%x", layouts);
+    SO_REQUIRE(!(layouts & SO_LAYOUT_IDX16) || n <= 65536u, "so_ellpack_upload: 16-bit columns need n <= 65536 (n = %u)", n);
 
     // Validate on the host before anything reaches a kernel: every stored slot must
     // name a column inside X, every count must fit the row.
@@ -509,6 +512,14 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
             }
         s = upload_array(ctx, WdT.data(), slots, &E->d_WdT);
         if (s == SO_OK) s = upload_array(ctx, idxT.data(), slots, &E->d_idxT);
+    }
+
+    if (s == SO_OK && (layouts & SO_LAYOUT_IDX16)) {
+        // The same slots as d_idx, two bytes each: so_matvec streams 6 bytes per nonzero instead of 8.
+        // Padding slots keep the low half of whatever they hold; no kernel uses them.
+        std::vector<uint16_t> idx16(slots);
+        for (size_t k = 0; k < slots; ++k) idx16[k] = (uint16_t)idx[k];
+        s = upload_array(ctx, idx16.data(), slots, &E->d_idx16);
     }
 
     if (s == SO_OK && (layouts & SO_LAYOUT_BINS)) {

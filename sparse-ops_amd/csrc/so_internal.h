@@ -17,6 +17,7 @@ struct so_tuning {
     int matmul_rbm = -1;     // SPARSEOPS_MATMUL_RBM: 0 forbids the row-block-merged kernel on handles that carry its layout, 1 forces it
     int matmul_rbm_split = 0;   // SPARSEOPS_MATMUL_RBM_SPLIT: 1, 2 or 4 workgroups per tile for RBM layouts built from now on
     int matvec_lanes = 0;    // SPARSEOPS_MATVEC_LANES: 8, 16, 32 or 64 lanes per row
+    int matvec_idx16 = -1;   // SPARSEOPS_MATVEC_IDX16: 0 keeps so_matvec on the 32-bit columns of a handle that has both
     int conv_min_cg = 0;     // SPARSEOPS_CONV_MIN_CG: fewest channel groups per workgroup a small grid may shrink to (16: never shrink)
     int conv_window = -1;    // SPARSEOPS_CONV_WINDOW: 1 forces the LDS-windowed kernel, 0 forbids it
     int conv_cpw = 0;        // SPARSEOPS_CONV_CPW: most output channels per wave
@@ -109,6 +110,7 @@ struct so_ellpack {
     uint32_t *d_nnz = nullptr;   // [m]
     float *d_WdT = nullptr;      // [r*m] slot-major (SO_LAYOUT_SLOT)
     uint32_t *d_idxT = nullptr;
+    uint16_t *d_idx16 = nullptr; // [m*r] the columns of d_idx in 16 bits (SO_LAYOUT_IDX16, n <= 65536)
     so_bin bins[3];              // SO_LAYOUT_BINS
     so_tiled tiled;              // SO_LAYOUT_TILED
     so_rbmm rbmm;                // SO_LAYOUT_RBM

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "libsparseops_hip.so")
 
 SO_OK, SO_ERR_NO_DEVICE, SO_ERR_INVALID, SO_ERR_OOM, SO_ERR_HIP, SO_ERR_BOUNDS = range(6)
 ACT = {"none": 0, "relu": 1, "sigmoid": 2, "tanh": 3}
-LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS, LAYOUT_TILED, LAYOUT_RBM = 1, 2, 4, 8, 16
+LAYOUT_ROW, LAYOUT_SLOT, LAYOUT_BINS, LAYOUT_TILED, LAYOUT_RBM, LAYOUT_IDX16 = 1, 2, 4, 8, 16, 32
 
 # Every symbol include/sparseops_hip.h declares.
 SYMBOLS = (
@@ -167,6 +167,12 @@ class DeviceEllpack:
         W = dW.download()
         dW.free()
         return W
+
+    def layouts(self):
+        """The mask of SO_LAYOUT_* the handle holds (so_ellpack_dims)."""
+        lay = ct.c_int()
+        self.ctx._ck(self.ctx.lib.so_ellpack_dims(self.h, None, None, None, None, ct.byref(lay)))
+        return lay.value
 
     def download(self, layout=LAYOUT_ROW):
         shape = (self.m, self.r) if layout == LAYOUT_ROW else (self.r, self.m)

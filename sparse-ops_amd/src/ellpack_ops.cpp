@@ -87,7 +87,10 @@ void ellpack_matvec(const Ellpack &E, const float *x, const float *bias, float *
     uint64_t total = 0;
     for (uint32_t c : E.nnz) total += c;
     const bool skewed = uint64_t(E.r) * E.m > 2 * total + E.m;
-    const so_ellpack *dE = mirror(E, skewed ? (SO_LAYOUT_ROW | SO_LAYOUT_BINS) : SO_LAYOUT_ROW);
+    // Up to 65536 columns fit 16 bits: the device keeps them that way as well and the product streams
+    // 6 bytes per nonzero instead of 8 (same bits).
+    const int compact = E.n <= 65536u ? SO_LAYOUT_IDX16 : 0;
+    const so_ellpack *dE = mirror(E, (skewed ? (SO_LAYOUT_ROW | SO_LAYOUT_BINS) : SO_LAYOUT_ROW) | compact);
     Staging &st = staging();
     st.x.reserve(std::size_t(E.n) * sizeof(float));
     st.y.reserve(std::size_t(E.m) * sizeof(float));

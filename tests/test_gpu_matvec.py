@@ -144,6 +144,87 @@ def test_matvec_degenerate(ctx):
         ctx.matvec(dE2, ctx.empty((32,)), None, ctx.empty((32,)), hipabi.LAYOUT_SLOT)   # layout not uploaded
 
 
+# ---- columns in 16 bits (SO_LAYOUT_IDX16): same kernels, 6 bytes per nonzero, same bits
+
+def both_column_widths(ctx, E, x, b, layouts, which):
+    """y from the handle's 16-bit columns and, on the same handle, from its 32-bit ones."""
+    dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, layouts | hipabi.LAYOUT_IDX16)
+    assert dE.layouts() & hipabi.LAYOUT_IDX16
+    dx, dy = ctx.array(x), ctx.empty((E.m,))
+    dB = ctx.array(b) if b is not None else None
+    out = {}
+    for lay in which:
+        dy.upload(np.full(E.m, np.nan, np.float32))
+        ctx.matvec(dE, dx, dB, dy, lay)
+        y16 = dy.download()
+        with ctx.tuning(SPARSEOPS_MATVEC_IDX16="0"):
+            dy.upload(np.full(E.m, np.nan, np.float32))
+            ctx.matvec(dE, dx, dB, dy, lay)
+        out[lay] = (y16, dy.download())
+    # the 32-bit arrays are untouched: the download is still the upload
+    Wd, idx, nnz = dE.download(hipabi.LAYOUT_ROW)
+    assert np.array_equal(Wd.view(np.uint32), E.Wd.view(np.uint32)) and np.array_equal(idx, E.idx) and np.array_equal(nnz, E.nnz)
+    dE.free()
+    return out
+
+
+@pytest.mark.parametrize("lanes", [0, 8, 16, 32, 64])
+@pytest.mark.parametrize("m,n,kmax", [(3001, 1000, 203), (517, 65536, 1300), (64, 300, 17), (20000, 256, 40), (300, 40000, 2600)])
+def test_matvec_16_bit_columns(ctx, lanes, m, n, kmax):
+    """Ragged rows (empty ones, odd r, rows of several passes, columns up to 65535) through the row kernel at
+    every lanes-per-row setting and through the binned kernel: the 16-bit columns give the bits of the 32-bit ones."""
+    rng = np.random.default_rng(lanes * 7 + m)
+    counts = np.minimum(rng.zipf(1.3, size=m) * 3, kmax)
+    counts[::7] = 0
+    counts[1] = kmax
+    cols = [np.sort(rng.choice(n, size=k, replace=False)).astype(np.uint32) for k in counts]
+    cols[1][-1] = n - 1                                    # the last column is used (65535 when n = 65536)
+    if kmax > 1:
+        cols[1][-2] = min(cols[1][-2], n - 2)
+    vals = [rng.standard_normal(k).astype(np.float32) for k in counts]
+    E = datagen.rows_to_ellpack(m, n, cols, vals)
+    x = rng.standard_normal(n).astype(np.float32)
+    b = rng.standard_normal(m).astype(np.float32)
+    y64 = b.astype(np.float64)
+    for i in range(m):
+        y64[i] += vals[i].astype(np.float64) @ x[cols[i]]
+    with ctx.tuning(SPARSEOPS_MATVEC_LANES=lanes or None):
+        res = both_column_widths(ctx, E, x, b, hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS, (hipabi.LAYOUT_ROW, hipabi.LAYOUT_BINS, 0))
+    for lay, (y16, y32) in res.items():
+        assert np.isfinite(y16).all(), lay
+        assert np.array_equal(y16, y32), lay
+        assert rel_err(y16, y64) <= TOL, lay
+
+
+def test_matvec_16_bit_columns_full_size(ctx, oracle):
+    """Configurations 2a and 2b with the compact columns: the oracle's result within tolerance, the 32-bit
+    kernels' bits."""
+    for gen, layouts, which in ((datagen.config2a, hipabi.LAYOUT_ROW, (hipabi.LAYOUT_ROW,)),
+                                (datagen.config2b, hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS, (hipabi.LAYOUT_BINS, hipabi.LAYOUT_ROW))):
+        E, x, b = gen()
+        yo = oracle.matvec(as_oracle(E), x, b)
+        for lay, (y16, y32) in both_column_widths(ctx, E, x, b, layouts, which).items():
+            assert np.array_equal(y16, y32), lay
+            assert rel_err(y16, yo) <= TOL, lay
+
+
+def test_matvec_16_bit_columns_need_few_columns(ctx):
+    W = np.zeros((4, 65537), np.float32)
+    W[2, 65536] = 1.0
+    E = datagen.encode_dense(W)
+    with pytest.raises(hipabi.SoError, match="65536"):
+        ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, hipabi.LAYOUT_ROW | hipabi.LAYOUT_IDX16)
+    # without the flag the same matrix is fine, and an empty one takes the flag
+    y = gpu_matvec(ctx, E, np.arange(65537, dtype=np.float32), None, layouts=hipabi.LAYOUT_ROW, which=(hipabi.LAYOUT_ROW,))
+    assert np.array_equal(y[hipabi.LAYOUT_ROW], [0, 0, 65536, 0])
+    E0 = datagen.encode_dense(np.zeros((3, 5), np.float32))
+    dE = ctx.upload_ellpack(E0.Wd, E0.idx, E0.nnz, 3, 5, E0.r, hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS | hipabi.LAYOUT_IDX16)
+    dy = ctx.array(np.full(3, np.nan, np.float32))
+    ctx.matvec(dE, ctx.array(np.ones(5, np.float32)), None, dy, 0)
+    assert np.array_equal(dy.download(), [0, 0, 0])
+    dE.free()
+
+
 # ---- the drop-in module: the reference's unit cases (tests/unit/test_matvec.py:12-46), seeded
 
 @pytest.mark.parametrize("m,n,sp", MATVEC_CASES)
