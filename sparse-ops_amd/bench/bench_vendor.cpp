@@ -273,6 +273,16 @@ int main(int argc, char **argv)
         report("Ellpack so_matvec (wave per row)", t_row, 0.0);
         const double t_bin = so_time([&] { SOCK(so_matvec(ctx, E_row, dX, nullptr, dY, SO_LAYOUT_BINS)); });
         report("Ellpack so_matvec (length bins)", t_bin, max_rel_diff(fetch(dY, size_t(M)), y_ref));
+        if (N <= 65536) {           // the same two kernels on a handle that also holds its columns in 16 bits
+            so_ellpack *E_c16 = nullptr;
+            SOCK(so_ellpack_upload(ctx, h.Wd.data(), h.idx.data(), h.nnz.data(), uint32_t(M), uint32_t(N), h.r,
+                                   SO_LAYOUT_ROW | SO_LAYOUT_BINS | SO_LAYOUT_IDX16, &E_c16));
+            const double t_row16 = so_time([&] { SOCK(so_matvec(ctx, E_c16, dX, nullptr, dY, SO_LAYOUT_ROW)); });
+            report("Ellpack so_matvec (wave per row, 16-bit columns)", t_row16, max_rel_diff(fetch(dY, size_t(M)), y_ref));
+            const double t_bin16 = so_time([&] { SOCK(so_matvec(ctx, E_c16, dX, nullptr, dY, SO_LAYOUT_BINS)); });
+            report("Ellpack so_matvec (length bins, 16-bit columns)", t_bin16, max_rel_diff(fetch(dY, size_t(M)), y_ref));
+            SOCK(so_ellpack_free(ctx, E_c16));
+        }
     }
 
     // --- rocSPARSE CSR ----------------------------------------------------------
