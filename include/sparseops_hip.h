@@ -74,10 +74,11 @@ enum { SO_ACT_NONE = 0, SO_ACT_RELU = 1, SO_ACT_SIGMOID = 2, SO_ACT_TANH = 3 };
  *        bit-identical to it, and are the same bits on every launch.  Rows may be in any
  *        order.  Costs about 1.4x the ROW arrays in HBM; with it so_matmul keeps a
  *        workspace in the context that grows on first use of a larger output.
- * IDX16: a second copy of the ROW layout's columns in 16 bits (needs n <= 65536; costs 2 bytes
- *        per slot).  so_matvec's ROW and BINS kernels then read 6 bytes per nonzero instead
- *        of 8 -- the product is a stream from HBM, so a quarter less time -- and give the same
- *        bits.  Nothing else reads it; downloads come from the 32-bit arrays. */
+ * IDX16: a second copy of the columns in 16 bits (needs n <= 65536; costs 2 bytes per slot,
+ *        and as much again for the SLOT copy when that is asked for too).  so_matvec then
+ *        reads 6 bytes per nonzero instead of 8 -- the product is a stream from HBM, so
+ *        about a fifth less time -- and gives the same bits.  Nothing else reads it;
+ *        downloads come from the 32-bit arrays. */
 enum { SO_LAYOUT_ROW = 1, SO_LAYOUT_SLOT = 2, SO_LAYOUT_BINS = 4, SO_LAYOUT_TILED = 8, SO_LAYOUT_RBM = 16, SO_LAYOUT_IDX16 = 32 };
 
 typedef struct so_ctx so_ctx;         /* one device + one stream + staging arena */
@@ -202,8 +203,8 @@ so_status so_matmul_reserve(so_ctx *ctx, const so_ellpack *E, uint32_t C);
 /* y[m] = E * x[n] + bias: ellpack_matvec (src/ellpack_matvec.cpp:20-147).
  * `layout` picks the kernel: SO_LAYOUT_ROW (one wave per row), SO_LAYOUT_SLOT
  * (one lane per row on the slot-major copy), SO_LAYOUT_BINS (length classes),
- * or 0 to let the library choose from what was uploaded.  The ROW and BINS kernels take
- * the columns from the SO_LAYOUT_IDX16 copy when the handle has one (same result). */
+ * or 0 to let the library choose from what was uploaded.  The kernels take the columns
+ * from the SO_LAYOUT_IDX16 copy when the handle has one (same result). */
 so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx,
                     const float *dBias, float *dy, int layout);
 

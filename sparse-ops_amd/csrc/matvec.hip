@@ -6,7 +6,7 @@
 // then never leave the CU), the pairs are read with 16-byte non-temporal loads,
 // four per lane in flight, and only the first nnz[i] slots of a row are touched,
 // so ELLPACK padding is never streamed.  A handle uploaded with SO_LAYOUT_IDX16 also has
-// its columns in 16 bits: the row-major kernels then stream 6 bytes per nonzero.
+// its columns in 16 bits: the kernels then stream 6 bytes per nonzero.
 //
 //   rows kernel    one wavefront per row on the row-major arrays; lanes take
 //                  aligned groups of four slots, partial sums are combined with a
@@ -298,9 +298,9 @@ void matvec_binned_kernel(const float *__restrict__ Wd, const void *__restrict__
     }
 }
 
-template <bool XLDS>
+template <bool XLDS, typename IdxT>
 __global__ __launch_bounds__(kBlock)
-void matvec_slot_kernel(const float *__restrict__ WdT, const uint32_t *__restrict__ idxT,
+void matvec_slot_kernel(const float *__restrict__ WdT, const IdxT *__restrict__ idxT,
                         const uint32_t *__restrict__ nnz, uint32_t m,
                         const float *__restrict__ x, uint32_t n,
                         const float *__restrict__ bias, float *__restrict__ y)
@@ -386,12 +386,18 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
 #undef SO_MV_ROWS
     } else if (layout == SO_LAYOUT_SLOT) {
         const uint32_t blocks = std::max(1u, std::min(so_ceil_div(E->m, kBlock), 2u * cus));
-        if (use_lds(ctx, matvec_slot_kernel<true>, E->n, E->total_nnz, blocks))
-            matvec_slot_kernel<true><<<blocks, kBlock, lds, ctx->stream>>>(E->d_WdT, E->d_idxT, E->d_nnz, E->m,
-                                                                           dx, E->n, dBias, dy);
-        else
-            matvec_slot_kernel<false><<<blocks, kBlock, 0, ctx->stream>>>(E->d_WdT, E->d_idxT, E->d_nnz, E->m,
-                                                                          dx, E->n, dBias, dy);
+#define SO_MV_SLOT(T, COLS)                                                                                        \
+        do {                                                                                                       \
+            if (use_lds(ctx, matvec_slot_kernel<true, T>, E->n, E->total_nnz, blocks))                             \
+                matvec_slot_kernel<true, T><<<blocks, kBlock, lds, ctx->stream>>>(E->d_WdT, COLS, E->d_nnz, E->m,  \
+                                                                                  dx, E->n, dBias, dy);            \
+            else                                                                                                   \
+                matvec_slot_kernel<false, T><<<blocks, kBlock, 0, ctx->stream>>>(E->d_WdT, COLS, E->d_nnz, E->m,   \
+                                                                                 dx, E->n, dBias, dy);             \
+        } while (0)
+        if (E->d_idxT16 && ctx->tune.matvec_idx16 != 0) SO_MV_SLOT(uint16_t, E->d_idxT16);
+        else SO_MV_SLOT(uint32_t, E->d_idxT);
+#undef SO_MV_SLOT
     } else {
         // One launch over the three length classes.  bins[] is ordered 4, 16, 64 lanes.
         BinArgs ba;

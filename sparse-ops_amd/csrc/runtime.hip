@@ -334,6 +334,7 @@ static void free_ellpack_arrays(so_ellpack *E)
     if (E->d_WdT) (void)hipFree(E->d_WdT);
     if (E->d_idxT) (void)hipFree(E->d_idxT);
     if (E->d_idx16) (void)hipFree(E->d_idx16);
+    if (E->d_idxT16) (void)hipFree(E->d_idxT16);
     for (auto &b : E->bins)
         if (b.d_rows) (void)hipFree(b.d_rows);
     if (E->tiled.d_entries) (void)hipFree(E->tiled.d_entries);
@@ -512,6 +513,11 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
             }
         s = upload_array(ctx, WdT.data(), slots, &E->d_WdT);
         if (s == SO_OK) s = upload_array(ctx, idxT.data(), slots, &E->d_idxT);
+        if (s == SO_OK && (layouts & SO_LAYOUT_IDX16)) {
+            std::vector<uint16_t> idxT16(slots);
+            for (size_t k = 0; k < slots; ++k) idxT16[k] = (uint16_t)idxT[k];
+            s = upload_array(ctx, idxT16.data(), slots, &E->d_idxT16);
+        }
     }
 
     if (s == SO_OK && (layouts & SO_LAYOUT_IDX16)) {

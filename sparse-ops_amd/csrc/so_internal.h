@@ -111,6 +111,7 @@ struct so_ellpack {
     float *d_WdT = nullptr;      // [r*m] slot-major (SO_LAYOUT_SLOT)
     uint32_t *d_idxT = nullptr;
     uint16_t *d_idx16 = nullptr; // [m*r] the columns of d_idx in 16 bits (SO_LAYOUT_IDX16, n <= 65536)
+    uint16_t *d_idxT16 = nullptr;// [r*m] the same for d_idxT (SO_LAYOUT_SLOT with SO_LAYOUT_IDX16)
     so_bin bins[3];              // SO_LAYOUT_BINS
     so_tiled tiled;              // SO_LAYOUT_TILED
     so_rbmm rbmm;                // SO_LAYOUT_RBM

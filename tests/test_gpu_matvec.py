@@ -172,7 +172,7 @@ def both_column_widths(ctx, E, x, b, layouts, which):
 @pytest.mark.parametrize("m,n,kmax", [(3001, 1000, 203), (517, 65536, 1300), (64, 300, 17), (20000, 256, 40), (300, 40000, 2600)])
 def test_matvec_16_bit_columns(ctx, lanes, m, n, kmax):
     """Ragged rows (empty ones, odd r, rows of several passes, columns up to 65535) through the row kernel at
-    every lanes-per-row setting and through the binned kernel: the 16-bit columns give the bits of the 32-bit ones."""
+    every lanes-per-row setting, through the binned kernel and the lane-per-row kernel: the 16-bit columns give the bits of the 32-bit ones."""
     rng = np.random.default_rng(lanes * 7 + m)
     counts = np.minimum(rng.zipf(1.3, size=m) * 3, kmax)
     counts[::7] = 0
@@ -189,7 +189,7 @@ def test_matvec_16_bit_columns(ctx, lanes, m, n, kmax):
     for i in range(m):
         y64[i] += vals[i].astype(np.float64) @ x[cols[i]]
     with ctx.tuning(SPARSEOPS_MATVEC_LANES=lanes or None):
-        res = both_column_widths(ctx, E, x, b, hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS, (hipabi.LAYOUT_ROW, hipabi.LAYOUT_BINS, 0))
+        res = both_column_widths(ctx, E, x, b, ALL, (hipabi.LAYOUT_ROW, hipabi.LAYOUT_BINS, hipabi.LAYOUT_SLOT, 0))
     for lay, (y16, y32) in res.items():
         assert np.isfinite(y16).all(), lay
         assert np.array_equal(y16, y32), lay
