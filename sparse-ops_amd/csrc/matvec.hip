@@ -11,9 +11,10 @@
 //   rows kernel    one wavefront per row on the row-major arrays; lanes take
 //                  aligned groups of four slots, partial sums are combined with a
 //                  butterfly of lane exchanges.
-//   binned kernel  one launch over three length classes (skewed matrices): whole
-//                  waves for long rows, 16 or 4 lanes per row for short ones;
-//                  workgroups of the long class are dispatched first.
+//   binned kernel  one launch over four length classes (skewed matrices): a whole
+//                  workgroup for rows of more than 4096 nonzeros, whole waves for
+//                  long rows, 16 or 4 lanes per row for short ones; workgroups of
+//                  the long classes are dispatched first.
 //   slot kernel    one lane per row on the slot-major arrays (consecutive rows'
 //                  k-th nonzeros are contiguous, so loads coalesce across lanes).
 //
@@ -239,10 +240,12 @@ __device__ __forceinline__ void short_rows(const float *__restrict__ Wd, const I
 }
 
 struct BinArgs {
-    const uint2 *rows64, *rows16, *rows4;      // (row, nonzeros of the row) per length class
-    uint32_t n64, n16, n4;                     // rows per class
-    uint32_t b64, b16;                         // workgroups given to the 64- and 16-lane classes
+    const uint2 *rowswg, *rows64, *rows16, *rows4;   // (row, nonzeros of the row) per length class
+    uint32_t nwg, n64, n16, n4;                      // rows per class
+    uint32_t bwg, b64, b16;                          // workgroups given to the workgroup-, 64- and 16-lane classes
 };
+
+constexpr uint32_t kBinnedTailBytes = 64;            // behind x in LDS: the 16 waves' partial sums of a workgroup-wide row
 
 template <bool XLDS, bool I16>
 __global__ __launch_bounds__(kBlock, 8)          // 64 registers: two workgroups per compute unit
@@ -251,7 +254,40 @@ void matvec_binned_kernel(const float *__restrict__ Wd, const void *__restrict__
                           const float *__restrict__ bias, float *__restrict__ y)
 {
     extern __shared__ float lds_x[];
-    const uint32_t b = blockIdx.x;
+    uint32_t b = blockIdx.x;
+    if (b < ba.bwg) {
+        // Rows of more than 4096 nonzeros: the 16 waves take the row's passes of 1024 slots in turn,
+        // the 16 partial sums meet in LDS (behind x) and are added in wave order.
+        const uint32_t lane = threadIdx.x & 63u;
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const f32x4 *Wd4 = reinterpret_cast<const f32x4 *>(Wd);
+        const typename ColGroup<I16>::T *idx4 = reinterpret_cast<const typename ColGroup<I16>::T *>(idxv);
+        float *part = lds_x + (XLDS ? ((n + 3u) & ~3u) : 0u);
+        const float *xs = stage_x<XLDS>(x, n, lds_x);
+        for (uint32_t g = b; g < ba.nwg; g += ba.bwg) {
+            const uint2 e = ba.rowswg[g];
+            const uint64_t beg = (uint64_t)e.x * r, end = beg + e.y;
+            const uint64_t qlast = (end - 1) >> 2;                  // e.y > 4096
+            float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+            for (uint64_t q = (beg >> 2) + wave * 256u + lane; q <= qlast; q += 256u * kWavesPerBlock) {
+                RowLoads<I16> L;
+                row_issue<64, I16>(Wd4, idx4, beg, end, q, L);
+                row_consume<64, I16>(L, beg, end, q, xs, a0, a1, a2, a3);
+            }
+            const float s = group_sum<64>((a0 + a1) + (a2 + a3));
+            if (lane == 0) part[wave] = s;
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                float t = part[0];
+#pragma unroll
+                for (int w = 1; w < kWavesPerBlock; ++w) t += part[w];
+                y[e.x] = (bias ? bias[e.x] : 0.0f) + t;
+            }
+            __syncthreads();                                        // part[] is reused by the next row
+        }
+        return;
+    }
+    b -= ba.bwg;
     if (b < ba.b64) {
         // A wave's first row (its only one unless the class has more rows than the launch has waves):
         // where it is and how long comes in one load, issued before x is staged.  The row itself is
@@ -293,7 +329,7 @@ void matvec_binned_kernel(const float *__restrict__ Wd, const void *__restrict__
         short_rows<XLDS, 16, 8>(Wd, idx, ba.rows16, ba.n16, b - ba.b64, ba.b16, r, x, n, lds_x, bias, y);
     } else {
         const typename ColGroup<I16>::E *idx = reinterpret_cast<const typename ColGroup<I16>::E *>(idxv);
-        short_rows<XLDS, 4, 4>(Wd, idx, ba.rows4, ba.n4, b - ba.b64 - ba.b16, gridDim.x - ba.b64 - ba.b16, r, x, n,
+        short_rows<XLDS, 4, 4>(Wd, idx, ba.rows4, ba.n4, b - ba.b64 - ba.b16, gridDim.x - ba.bwg - ba.b64 - ba.b16, r, x, n,
                                lds_x, bias, y);
     }
 }
@@ -322,10 +358,10 @@ void matvec_slot_kernel(const float *__restrict__ WdT, const IdxT *__restrict__ 
 // LDS staging of x is worth its per-workgroup copy only when a workgroup then
 // serves many nonzeros from it; it needs n floats of LDS (set up once per kernel).
 template <typename K>
-bool use_lds(so_ctx *ctx, K kernel, uint32_t n, uint64_t nnz_total, uint32_t blocks)
+bool use_lds(so_ctx *ctx, K kernel, uint32_t n, uint64_t nnz_total, uint32_t blocks, size_t extra = 0)
 {
-    const size_t lds = (size_t)n * sizeof(float);
-    if (lds == 0 || lds > (size_t)ctx->max_lds_bytes) return false;
+    const size_t lds = (size_t)n * sizeof(float) + extra;
+    if (n == 0 || lds > (size_t)ctx->max_lds_bytes) return false;
     if (nnz_total < (uint64_t)n * blocks) return false;   // fewer gathers than staged elements
     if (lds > 48 * 1024 && so_allow_big_lds(ctx, (const void *)kernel) != hipSuccess) return false;
     return true;
@@ -399,24 +435,28 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
         else SO_MV_SLOT(uint32_t, E->d_idxT);
 #undef SO_MV_SLOT
     } else {
-        // One launch over the three length classes.  bins[] is ordered 4, 16, 64 lanes.
+        // One launch over the four length classes.  bins[] is ordered 4, 16, 64 lanes, workgroup.
         BinArgs ba;
+        ba.rowswg = reinterpret_cast<const uint2 *>(E->bins[3].d_rows);  ba.nwg = E->bins[3].count;
+        ba.bwg = std::min(ba.nwg, cus);
         ba.rows4 = reinterpret_cast<const uint2 *>(E->bins[0].d_rows);   ba.n4 = E->bins[0].count;
         ba.rows16 = reinterpret_cast<const uint2 *>(E->bins[1].d_rows);  ba.n16 = E->bins[1].count;
         ba.rows64 = reinterpret_cast<const uint2 *>(E->bins[2].d_rows);  ba.n64 = E->bins[2].count;
         ba.b64 = std::min(so_ceil_div(ba.n64, kWavesPerBlock), 2u * cus);
         ba.b16 = std::min(so_ceil_div(ba.n16, kBlock / 16), std::max(1u, cus / 4));
         const uint32_t b4 = std::min(so_ceil_div(ba.n4, kBlock / 4), std::max(1u, cus / 4));
-        const uint32_t blocks = ba.b64 + ba.b16 + b4;
+        const uint32_t blocks = ba.bwg + ba.b64 + ba.b16 + b4;
         if (blocks == 0) return SO_OK;
+        // x padded to whole 16-byte groups, then the partial sums of a workgroup-wide row
+        const size_t lds_tail = (((size_t)E->n + 3) & ~(size_t)3) * sizeof(float) + kBinnedTailBytes;
 #define SO_MV_BINNED(I16)                                                                                          \
         do {                                                                                                       \
-            if (use_lds(ctx, matvec_binned_kernel<true, I16>, E->n, E->total_nnz, blocks))                         \
-                matvec_binned_kernel<true, I16><<<blocks, kBlock, lds, ctx->stream>>>(E->d_Wd, cols, ba, E->r,     \
-                                                                                      dx, E->n, dBias, dy);        \
+            if (use_lds(ctx, matvec_binned_kernel<true, I16>, E->n, E->total_nnz, blocks, lds_tail - lds))         \
+                matvec_binned_kernel<true, I16><<<blocks, kBlock, lds_tail, ctx->stream>>>(E->d_Wd, cols, ba, E->r, \
+                                                                                           dx, E->n, dBias, dy);   \
             else                                                                                                   \
-                matvec_binned_kernel<false, I16><<<blocks, kBlock, 0, ctx->stream>>>(E->d_Wd, cols, ba, E->r,      \
-                                                                                     dx, E->n, dBias, dy);         \
+                matvec_binned_kernel<false, I16><<<blocks, kBlock, kBinnedTailBytes, ctx->stream>>>(               \
+                    E->d_Wd, cols, ba, E->r, dx, E->n, dBias, dy);                                                 \
         } while (0)
         if (i16) SO_MV_BINNED(true);
         else SO_MV_BINNED(false);

@@ -529,18 +529,19 @@ extern "C" so_status so_ellpack_upload(so_ctx *ctx, const float *Wd, const uint3
     }
 
     if (s == SO_OK && (layouts & SO_LAYOUT_BINS)) {
-        // Length classes: <= 16 nonzeros -> 4 lanes per row, <= 128 -> 16 lanes,
-        // longer -> a whole wave.  Long rows first inside a class, so the last
-        // waves to start are the short ones.
-        static const uint32_t group[3] = {4, 16, 64};
-        static const uint32_t limit[3] = {16, 128, 0xffffffffu};
-        std::vector<uint32_t> rows[3];
+        // Length classes: <= 16 nonzeros -> 4 lanes per row, <= 128 -> 16 lanes, <= 4096 -> a whole
+        // wave, longer -> a whole workgroup (a single wave would walk such a row long after every
+        // other row is done).  Long rows first inside a class, so the last waves to start are the
+        // short ones.
+        static const uint32_t group[4] = {4, 16, 64, 1024};
+        static const uint32_t limit[4] = {16, 128, 4096, 0xffffffffu};
+        std::vector<uint32_t> rows[4];
         for (uint32_t i = 0; i < m; ++i) {
             int b = 0;
             while (nnz[i] > limit[b]) ++b;
             rows[b].push_back(i);
         }
-        for (int b = 0; b < 3 && s == SO_OK; ++b) {
+        for (int b = 0; b < 4 && s == SO_OK; ++b) {
             std::stable_sort(rows[b].begin(), rows[b].end(),
                              [&](uint32_t a, uint32_t c) { return nnz[a] > nnz[c]; });
             E->bins[b].group = group[b];

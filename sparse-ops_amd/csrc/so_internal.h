@@ -52,7 +52,7 @@ struct so_ctx {
 
 // Rows of one length class for the binned matvec: `group` lanes cooperate on a row.
 struct so_bin {
-    uint32_t group = 0;      // 4, 16 or 64 lanes per row
+    uint32_t group = 0;      // 4, 16 or 64 lanes per row, 1024: a whole workgroup
     uint32_t count = 0;      // rows in this class
     uint32_t *d_rows = nullptr;   // count pairs (row, nonzeros of the row), longest rows first
 };
@@ -112,7 +112,7 @@ struct so_ellpack {
     uint32_t *d_idxT = nullptr;
     uint16_t *d_idx16 = nullptr; // [m*r] the columns of d_idx in 16 bits (SO_LAYOUT_IDX16, n <= 65536)
     uint16_t *d_idxT16 = nullptr;// [r*m] the same for d_idxT (SO_LAYOUT_SLOT with SO_LAYOUT_IDX16)
-    so_bin bins[3];              // SO_LAYOUT_BINS
+    so_bin bins[4];              // SO_LAYOUT_BINS
     so_tiled tiled;              // SO_LAYOUT_TILED
     so_rbmm rbmm;                // SO_LAYOUT_RBM
 };

@@ -225,6 +225,39 @@ def test_matvec_16_bit_columns_need_few_columns(ctx):
     dE.free()
 
 
+@pytest.mark.parametrize("n,long_rows", [(20000, (20000, 4097, 9000)), (70000, (70000, 33000)), (5000, (5000,) * 40)])
+def test_matvec_binned_very_long_rows(ctx, n, long_rows):
+    """Rows of more than 4096 nonzeros get a whole workgroup in the binned kernel (16 waves share the row, their
+    partial sums meet in LDS): a few such rows among short ones, a fully dense row, more such rows than the launch
+    has workgroups for them at once would need, x staged in LDS or not, both column widths."""
+    rng = np.random.default_rng(n)
+    m = 700
+    counts = np.minimum(rng.zipf(1.4, size=m) * 2, 300)
+    counts[::9] = 0
+    where = rng.choice(m, size=len(long_rows), replace=False)
+    counts[where] = long_rows
+    cols = [np.sort(rng.choice(n, size=k, replace=False)).astype(np.uint32) for k in counts]
+    vals = [rng.standard_normal(k).astype(np.float32) for k in counts]
+    E = datagen.rows_to_ellpack(m, n, cols, vals)
+    x = rng.standard_normal(n).astype(np.float32)
+    b = rng.standard_normal(m).astype(np.float32)
+    y64 = b.astype(np.float64)
+    for i in range(m):
+        y64[i] += vals[i].astype(np.float64) @ x[cols[i]]
+    lay = hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS
+    if n <= 65536:
+        for which, (y16, y32) in both_column_widths(ctx, E, x, b, lay, (hipabi.LAYOUT_BINS, hipabi.LAYOUT_ROW)).items():
+            assert np.isfinite(y16).all() and np.array_equal(y16, y32), which
+            assert rel_err(y16, y64) <= TOL, which
+    else:
+        for which, y in gpu_matvec(ctx, E, x, b, layouts=lay, which=(hipabi.LAYOUT_BINS, hipabi.LAYOUT_ROW)).items():
+            assert np.isfinite(y).all() and rel_err(y, y64) <= TOL, which
+    # the same launch twice gives the same bits (the partial sums are added in a fixed order)
+    y1 = gpu_matvec(ctx, E, x, b, layouts=lay, which=(hipabi.LAYOUT_BINS,))[hipabi.LAYOUT_BINS]
+    y2 = gpu_matvec(ctx, E, x, b, layouts=lay, which=(hipabi.LAYOUT_BINS,))[hipabi.LAYOUT_BINS]
+    assert np.array_equal(y1, y2)
+
+
 # ---- the drop-in module: the reference's unit cases (tests/unit/test_matvec.py:12-46), seeded
 
 @pytest.mark.parametrize("m,n,sp", MATVEC_CASES)
