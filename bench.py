@@ -43,7 +43,7 @@ LDS_OPERAND_PEAK_TF = 78.6   # 256 CUs x 256 B/clk of ds_read_b128 (measured 255
 TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
 HEADLINE_KERNEL = "ellpack_matmul_rbm_kernel<0>"
 TILED_KERNEL = "ellpack_matmul_tiled_kernel<0>"
-MATVEC_KERNELS = {"ellpack_matvec 16384x16384, 95% Bernoulli": ("matvec_rows_kernel<true,64,true>", "matvec 16384^2 uniform"),
+MATVEC_KERNELS = {"ellpack_matvec 16384x16384, 95% Bernoulli": ("matvec_binned_kernel<true,true>", "matvec 16384^2 uniform"),
                   "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048": ("matvec_binned_kernel<true,true>", "matvec 16384^2 zipf")}
 
 
@@ -223,10 +223,14 @@ def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup
     # Up to 65536 columns the handle also keeps them in 16 bits (SO_LAYOUT_IDX16) and so_matvec streams 6 bytes
     # per nonzero instead of the format's 8: same bits, a quarter less to read.  `alg_bytes` and `hbm_frac` stay
     # on the reference format's 8 bytes per nonzero; `bytes_read` / `hbm_frac_bytes_read` are what the kernel
-    # actually streams, and `idx32` is the same handle with the 32-bit columns.
+    # actually streams, and `idx32` is the same handle with the 32-bit columns.  As the host layer does
+    # (ellpack_matvec), compact columns go with the length-class kernel, which on them is the faster one for even
+    # rows too; `idx32` runs the kernel the host layer takes without them (`layout`).
     compact = E.n <= 65536
+    layout32 = layout
     if compact:
-        layouts |= hipabi.LAYOUT_IDX16
+        layouts |= hipabi.LAYOUT_IDX16 | hipabi.LAYOUT_BINS
+        layout = hipabi.LAYOUT_BINS
     dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, layouts)
     dx, dB, dy = ctx.array(x), ctx.array(b), ctx.empty((E.m,))
     _, ms = time_launches(ctx, lambda: ctx.matvec(dE, dx, dB, dy, layout), steps, warmup)
@@ -235,7 +239,8 @@ def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup
     nread = (6 if compact else 8) * E.total_nnz + vectors
     out = {"workload": name, "m": E.m, "n": E.n, "r": E.r, "nnz": E.total_nnz, "us_per_launch": round(ms * 1e3, 2),
            "alg_bytes": nbytes, "GBps": round(nbytes / ms / 1e6, 1), "hbm_frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
-           "column_bits": 16 if compact else 32, "bytes_read": nread,
+           "column_bits": 16 if compact else 32, "kernel": "length classes" if layout == hipabi.LAYOUT_BINS else "wave per row",
+           "bytes_read": nread,
            "hbm_frac_bytes_read": round(nread / ms / 1e6 / HBM_PEAK_GBS, 4),
            "padded_bytes": 8 * E.m * E.r,
            "traffic": measured_traffic(*MATVEC_KERNELS[name]) if name in MATVEC_KERNELS else None}
@@ -258,11 +263,15 @@ def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup
     out["cache_cold_copies"] = len(copies)
     if compact:
         y16 = dy.download()
+        def rotate32():
+            ctx.matvec(copies[turn[0] % len(copies)], dx, dB, dy, layout32)
+            turn[0] += 1
         with ctx.tuning(SPARSEOPS_MATVEC_IDX16="0"):
-            _, ms32 = time_launches(ctx, lambda: ctx.matvec(dE, dx, dB, dy, layout), steps, warmup)
-            _, cold32 = time_launches(ctx, rotate, cold_steps, len(copies))
+            _, ms32 = time_launches(ctx, lambda: ctx.matvec(dE, dx, dB, dy, layout32), steps, warmup)
+            _, cold32 = time_launches(ctx, rotate32, cold_steps, len(copies))
             ctx.matvec(dE, dx, dB, dy, layout)
-        out["idx32"] = {"us_per_launch": round(ms32 * 1e3, 2), "hbm_frac": round(nbytes / ms32 / 1e6 / HBM_PEAK_GBS, 4),
+        out["idx32"] = {"kernel": "length classes" if layout32 == hipabi.LAYOUT_BINS else "wave per row",
+                        "us_per_launch": round(ms32 * 1e3, 2), "hbm_frac": round(nbytes / ms32 / 1e6 / HBM_PEAK_GBS, 4),
                         "us_per_launch_cache_cold": round(cold32 * 1e3, 2),
                         "hbm_frac_cache_cold": round(nbytes / cold32 / 1e6 / HBM_PEAK_GBS, 4),
                         "same_bits_as_16_bit_columns": bool(np.array_equal(y16, dy.download()))}
@@ -407,8 +416,8 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip matvec and MLP measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline")
     ap.add_argument("--skip-extra", action="append", default=[], metavar="NAME",
-                    help="leave out one entry of `extras` (e.g. matvec_uniform_65536_rows, which runs the same kernel as "
-                         "matvec_uniform: counter passes that average per kernel name need the two apart); repeatable")
+                    help="leave out one entry of `extras` (e.g. matvec_uniform_65536_rows and matvec_zipf, which run the same "
+                         "kernel as matvec_uniform: counter passes that average per kernel name need them apart); repeatable")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain 256 MiB copy kernel (scale factor for rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -523,23 +532,27 @@ def main():
         for a in (dX1, dB1, dY1):
             a.free()
         dE1.free()
-        log("matvec 16384^2 uniform ...")
-        extras["matvec_uniform"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 16384x16384, 95% Bernoulli",
-                                                datagen.config2a, hipabi.LAYOUT_ROW, hipabi.LAYOUT_ROW, k, args.warmup, not args.no_cpu)
-        log("matvec 16384^2 zipf ...")
-        extras["matvec_zipf"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048",
-                                             datagen.config2b, hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS, hipabi.LAYOUT_BINS,
-                                             k, args.warmup, not args.no_cpu)
+        if "matvec_uniform" not in args.skip_extra:
+            log("matvec 16384^2 uniform ...")
+            extras["matvec_uniform"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 16384x16384, 95% Bernoulli",
+                                                    datagen.config2a, hipabi.LAYOUT_ROW, hipabi.LAYOUT_ROW, k, args.warmup, not args.no_cpu)
+        if "matvec_zipf" not in args.skip_extra:
+            log("matvec 16384^2 zipf ...")
+            extras["matvec_zipf"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 16384x16384, Zipf(1.2) rows capped at 2048",
+                                                 datagen.config2b, hipabi.LAYOUT_ROW | hipabi.LAYOUT_BINS, hipabi.LAYOUT_BINS,
+                                                 k, args.warmup, not args.no_cpu)
         if "matvec_uniform_65536_rows" not in args.skip_extra:
             log("matvec 65536x16384 uniform ...")
             # four times the rows of config 2a: what the same kernel streams once its fixed per-launch cost is amortised
             extras["matvec_uniform_65536_rows"] = bench_matvec(ctx, hipabi, datagen, "ellpack_matvec 65536x16384, 95% Bernoulli",
                                                                lambda: datagen.uniform_ellpack(48, 65536, 16384, 0.05),
                                                                hipabi.LAYOUT_ROW, hipabi.LAYOUT_ROW, max(10, k // 4), 3, False)
-        log("sparse MLP ...")
-        extras["mlp"] = bench_mlp(k, args.warmup, with_cpu=not args.no_cpu)
-        log("sparse CNN ...")
-        extras["cnn"] = bench_cnn(max(10, args.steps // 10), 5, with_cpu=not args.no_cpu)
+        if "mlp" not in args.skip_extra:
+            log("sparse MLP ...")
+            extras["mlp"] = bench_mlp(k, args.warmup, with_cpu=not args.no_cpu)
+        if "cnn" not in args.skip_extra:
+            log("sparse CNN ...")
+            extras["cnn"] = bench_cnn(max(10, args.steps // 10), 5, with_cpu=not args.no_cpu)
         result["extras"] = extras
     ctx.close()
     print(json.dumps(result), flush=True)
