@@ -225,12 +225,14 @@ def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup
     # on the reference format's 8 bytes per nonzero; `bytes_read` / `hbm_frac_bytes_read` are what the kernel
     # actually streams, and `idx32` is the same handle with the 32-bit columns.  As the host layer does
     # (ellpack_matvec), compact columns go with the length-class kernel, which on them is the faster one for even
-    # rows too; `idx32` runs the kernel the host layer takes without them (`layout`).
+    # rows too while a wave gets only a few rows; `idx32` runs the kernel the host layer takes without them.
     compact = E.n <= 65536
     layout32 = layout
     if compact:
-        layouts |= hipabi.LAYOUT_IDX16 | hipabi.LAYOUT_BINS
-        layout = hipabi.LAYOUT_BINS
+        layouts |= hipabi.LAYOUT_IDX16
+        if E.m <= 64 * ctx.info()[1]:          # so_matvec's own rule (layout 0): few rows per wave
+            layouts |= hipabi.LAYOUT_BINS
+            layout = hipabi.LAYOUT_BINS
     dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, layouts)
     dx, dB, dy = ctx.array(x), ctx.array(b), ctx.empty((E.m,))
     _, ms = time_launches(ctx, lambda: ctx.matvec(dE, dx, dB, dy, layout), steps, warmup)

@@ -377,7 +377,13 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
     SO_REQUIRE(dy != nullptr, "so_matvec: y is null");
     SO_REQUIRE(dx != nullptr || E->total_nnz == 0, "so_matvec: x is null");
     if (layout == 0) {
-        if (E->layouts & SO_LAYOUT_BINS) layout = SO_LAYOUT_BINS;
+        // Length classes for skewed rows (the widest row far above the mean), and for even rows on 16-bit columns
+        // while a wave gets only a few of them (two workgroups per compute unit fit there; measured 16384 rows of
+        // 820 nonzeros: 15.0 against 15.6 us) -- with many rows per wave the row kernel, which requests a wave's
+        // next row while it sums the current one, is ahead (65536 rows: 51 against 56 us).
+        const bool skewed = (uint64_t)E->r * E->m > 2 * E->total_nnz + E->m;
+        const bool few_rows = E->d_idx16 != nullptr && ctx->tune.matvec_idx16 != 0 && E->m <= 64u * (uint32_t)ctx->compute_units;
+        if ((E->layouts & SO_LAYOUT_BINS) && (skewed || few_rows)) layout = SO_LAYOUT_BINS;
         else if ((E->layouts & SO_LAYOUT_SLOT) && E->max_nnz <= 64) layout = SO_LAYOUT_SLOT;
         else layout = SO_LAYOUT_ROW;
     }

@@ -88,12 +88,10 @@ void ellpack_matvec(const Ellpack &E, const float *x, const float *bias, float *
     for (uint32_t c : E.nnz) total += c;
     const bool skewed = uint64_t(E.r) * E.m > 2 * total + E.m;
     // Up to 65536 columns fit 16 bits: the device keeps them that way as well and the product streams
-    // 6 bytes per nonzero instead of 8 (same bits).
-    // On those the length-class kernel is the faster one for even rows too (two workgroups per compute unit
-    // fit: 16384 x 16384 at 95 % sparsity 15.0 against 15.6 us); on 32-bit columns the wave-per-row kernel is.
+    // 6 bytes per nonzero instead of 8 (same bits).  On those the length-class kernel is the faster one for
+    // even rows too while a wave gets only a few rows; so_matvec chooses between the two (layout 0).
     const int compact = E.n <= 65536u ? SO_LAYOUT_IDX16 : 0;
-    const bool binned = skewed || compact;
-    const so_ellpack *dE = mirror(E, (binned ? (SO_LAYOUT_ROW | SO_LAYOUT_BINS) : SO_LAYOUT_ROW) | compact);
+    const so_ellpack *dE = mirror(E, ((skewed || compact) ? (SO_LAYOUT_ROW | SO_LAYOUT_BINS) : SO_LAYOUT_ROW) | compact);
     Staging &st = staging();
     st.x.reserve(std::size_t(E.n) * sizeof(float));
     st.y.reserve(std::size_t(E.m) * sizeof(float));
@@ -104,6 +102,6 @@ void ellpack_matvec(const Ellpack &E, const float *x, const float *bias, float *
         check(so_h2d(ctx, st.bias.get(), bias, std::size_t(E.m) * sizeof(float)), "so_h2d(bias)");
         dBias = st.bias.f32();
     }
-    check(so_matvec(ctx, dE, st.x.f32(), dBias, st.y.f32(), binned ? SO_LAYOUT_BINS : SO_LAYOUT_ROW), "so_matvec");
+    check(so_matvec(ctx, dE, st.x.f32(), dBias, st.y.f32(), 0), "so_matvec");
     check(so_d2h(ctx, y, st.y.get(), std::size_t(E.m) * sizeof(float)), "so_d2h(y)");
 }
