@@ -230,7 +230,7 @@ def bench_matvec(ctx, hipabi, datagen, name, gen, layouts, layout, steps, warmup
     layout32 = layout
     if compact:
         layouts |= hipabi.LAYOUT_IDX16
-        if E.m <= 64 * ctx.info()[1]:          # so_matvec's own rule (layout 0): few rows per wave
+        if 4 <= E.m // (16 * ctx.info()[1]) < 6:          # so_matvec's own rule (layout 0): two or three rows per wave
             layouts |= hipabi.LAYOUT_BINS
             layout = hipabi.LAYOUT_BINS
     dE = ctx.upload_ellpack(E.Wd, E.idx, E.nnz, E.m, E.n, E.r, layouts)

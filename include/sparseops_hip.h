@@ -204,7 +204,7 @@ so_status so_matmul_reserve(so_ctx *ctx, const so_ellpack *E, uint32_t C);
  * `layout` picks the kernel: SO_LAYOUT_ROW (one wave per row), SO_LAYOUT_SLOT
  * (one lane per row on the slot-major copy), SO_LAYOUT_BINS (length classes),
  * or 0 to let the library choose from what was uploaded (length classes for skewed rows
- * and, on 16-bit columns, for matrices of up to 64 rows per compute unit; the lane-per-row
+ * and, on 16-bit columns, for matrices of 64 to 96 rows per compute unit; the lane-per-row
  * kernel for rows of at most 64 nonzeros; else one wave per row).  The kernels take the columns
  * from the SO_LAYOUT_IDX16 copy when the handle has one (same result). */
 so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx,

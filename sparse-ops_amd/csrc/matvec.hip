@@ -377,12 +377,14 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
     SO_REQUIRE(dy != nullptr, "so_matvec: y is null");
     SO_REQUIRE(dx != nullptr || E->total_nnz == 0, "so_matvec: x is null");
     if (layout == 0) {
-        // Length classes for skewed rows (the widest row far above the mean), and for even rows on 16-bit columns
-        // while a wave gets only a few of them (two workgroups per compute unit fit there; measured 16384 rows of
-        // 820 nonzeros: 15.0 against 15.6 us) -- with many rows per wave the row kernel, which requests a wave's
-        // next row while it sums the current one, is ahead (65536 rows: 51 against 56 us).
+        // Length classes for skewed rows (the widest row far above the mean).  For even rows the row kernel, which
+        // requests a wave's next row while it sums the current one, is the better one except on 16-bit columns
+        // where the length-class launch fills its two workgroups per compute unit with two or three rows per wave
+        // (16384 columns, 820 nonzeros per row; rows / us row kernel / us length classes: 8192 / 9.3 / 10.1,
+        // 16384 / 15.6 / 15.0, 24576 / 21.7 / 21.7, 32768 / 27.5 / 28.3, 49152 / 39.3 / 42.4, 65536 / 51 / 56).
         const bool skewed = (uint64_t)E->r * E->m > 2 * E->total_nnz + E->m;
-        const bool few_rows = E->d_idx16 != nullptr && ctx->tune.matvec_idx16 != 0 && E->m <= 64u * (uint32_t)ctx->compute_units;
+        const uint32_t per_wave_x2 = E->m / (16u * (uint32_t)ctx->compute_units);           // rows per wave of 2 x CUs workgroups, doubled
+        const bool few_rows = E->d_idx16 != nullptr && ctx->tune.matvec_idx16 != 0 && per_wave_x2 >= 4 && per_wave_x2 < 6;
         if ((E->layouts & SO_LAYOUT_BINS) && (skewed || few_rows)) layout = SO_LAYOUT_BINS;
         else if ((E->layouts & SO_LAYOUT_SLOT) && E->max_nnz <= 64) layout = SO_LAYOUT_SLOT;
         else layout = SO_LAYOUT_ROW;
@@ -451,6 +453,15 @@ extern "C" so_status so_matvec(so_ctx *ctx, const so_ellpack *E, const float *dx
         ba.b64 = std::min(so_ceil_div(ba.n64, kWavesPerBlock), 2u * cus);
         ba.b16 = std::min(so_ceil_div(ba.n16, kBlock / 16), std::max(1u, cus / 4));
         const uint32_t b4 = std::min(so_ceil_div(ba.n4, kBlock / 4), std::max(1u, cus / 4));
+        // Staging x pays while a workgroup gathers at least as many elements as it stages (use_lds): rather than
+        // give that up, a launch with few nonzeros per workgroup takes fewer workgroups of the wave-per-row class,
+        // down to one per compute unit (8192 rows of 820 nonzeros: 20.8 us unstaged on 512 workgroups).
+        if (E->n > 0) {
+            const uint64_t pays = E->total_nnz / E->n;                       // workgroups for which staging pays
+            const uint32_t others = ba.bwg + ba.b16 + b4;
+            if ((uint64_t)others + ba.b64 > pays && ba.b64 > cus)
+                ba.b64 = (uint32_t)std::max<uint64_t>(cus, pays > others ? pays - others : 0);
+        }
         const uint32_t blocks = ba.bwg + ba.b64 + ba.b16 + b4;
         if (blocks == 0) return SO_OK;
         // x padded to whole 16-byte groups, then the partial sums of a workgroup-wide row
