@@ -211,6 +211,7 @@ __device__ __forceinline__ void short_rows(const float *__restrict__ Wd, const I
     const uint32_t stride = blocks * (kBlock / G);
     uint32_t g = block * (kBlock / G) + threadIdx.x / G;
     const uint2 e = g < count ? rows[g] : make_uint2(0u, 0u);
+    uint2 en = g + stride < count ? rows[g + stride] : make_uint2(0u, 0u);     // the group's next task, a row ahead
     const uint64_t base = (uint64_t)e.x * r;
     float w[T];
     uint32_t c[T];
@@ -233,9 +234,10 @@ __device__ __forceinline__ void short_rows(const float *__restrict__ Wd, const I
         if (sub == 0) y[e.x] = (bias ? bias[e.x] : 0.0f) + a;
     }
     for (g += stride; g < count; g += stride) {
-        const uint2 en = rows[g];
-        const float s = group_row_dot<G>(Wd, idx, (uint64_t)en.x * r, en.y, xs, sub);
-        if (sub == 0) y[en.x] = (bias ? bias[en.x] : 0.0f) + s;
+        const uint2 ec = en;
+        if (g + stride < count) en = rows[g + stride];
+        const float s = group_row_dot<G>(Wd, idx, (uint64_t)ec.x * r, ec.y, xs, sub);
+        if (sub == 0) y[ec.x] = (bias ? bias[ec.x] : 0.0f) + s;
     }
 }
 
@@ -299,6 +301,8 @@ void matvec_binned_kernel(const float *__restrict__ Wd, const void *__restrict__
         const typename ColGroup<I16>::T *idx4 = reinterpret_cast<const typename ColGroup<I16>::T *>(idxv);
         uint32_t g = __builtin_amdgcn_readfirstlane(b * kWavesPerBlock + (threadIdx.x >> 6));
         const uint2 e = g < ba.n64 ? ba.rows64[g] : make_uint2(0u, 0u);
+        // the wave's next task, requested a row ahead so that its row never waits for it
+        uint2 en = g + stride < ba.n64 ? ba.rows64[g + stride] : make_uint2(0u, 0u);
         const uint64_t beg = (uint64_t)e.x * r, end = beg + e.y;
         const uint64_t q0 = (beg >> 2) + lane;
         const float *xs = stage_x<XLDS>(x, n, lds_x);
@@ -319,10 +323,11 @@ void matvec_binned_kernel(const float *__restrict__ Wd, const void *__restrict__
             if (lane == 0) y[e.x] = (bias ? bias[e.x] : 0.0f) + s;
         }
         for (g += stride; g < ba.n64; g += stride) {
-            const uint2 en = ba.rows64[g];
-            const uint64_t nbeg = (uint64_t)en.x * r;
-            const float s = wave_row_dot<I16>(Wd4, idx4, nbeg, nbeg + en.y, xs, lane);
-            if (lane == 0) y[en.x] = (bias ? bias[en.x] : 0.0f) + s;
+            const uint2 ec = en;
+            if (g + stride < ba.n64) en = ba.rows64[g + stride];
+            const uint64_t nbeg = (uint64_t)ec.x * r;
+            const float s = wave_row_dot<I16>(Wd4, idx4, nbeg, nbeg + ec.y, xs, lane);
+            if (lane == 0) y[ec.x] = (bias ? bias[ec.x] : 0.0f) + s;
         }
     } else if (b < ba.b64 + ba.b16) {
         const typename ColGroup<I16>::E *idx = reinterpret_cast<const typename ColGroup<I16>::E *>(idxv);
