@@ -69,8 +69,16 @@ struct WinArgs {
     uint32_t sth, stw;  // window pixels between neighbouring output pixels
     uint32_t sbh, sbw;  // input pixels between neighbouring window pixels
     uint32_t order[16]; // slot -> output pixel of the tile (ty * TW + tx), one byte per slot; see window_pixel_order
+    uint32_t mIW, mIH, mTW, mTilesX, mPg;   // window_magic of IW, IH, TW, tiles_x and pg: the kernels' index arithmetic divides by them
     so_lds::wait_status ws;   // bounded waits on the progress counters
 };
+
+// x / d for the small operands of the window index arithmetic (x * d < 2^32: window elements and
+// pixels count a few thousand, the divisors are window or tile extents) as one multiply-high by
+// M = ceil(2^32 / d) instead of the ~25 instructions of a general 32-bit division: exact, because
+// M * d - 2^32 < d makes the error of x * M / 2^32 smaller than 1 / d.  d == 1 has no 32-bit M.
+inline uint32_t window_magic(uint32_t d) { return d > 1 ? (uint32_t)(((1ull << 32) + d - 1) / d) : 0u; }
+__device__ __forceinline__ uint32_t window_div(uint32_t x, uint32_t d, uint32_t M) { return d == 1u ? x : __umulhi(x, M); }
 
 // Along an axis on which the kernel has a single tap, a strided convolution reads only every
 // stride-th input pixel: the window then holds just those (one window pixel per output pixel)

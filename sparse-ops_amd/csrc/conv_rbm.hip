@@ -236,8 +236,9 @@ void conv2d_rbm_kernel(const int4 *__restrict__ sets, const uint32_t *__restrict
     constexpr uint32_t BT = LPP * 4, PPW = 64 / LPP, SHIFT = (LPP == 4 ? 6 : LPP == 2 ? 5 : 4);
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t pgi = wave % a.pg, cgi = wave / a.pg;
-    const uint32_t th0 = (blockIdx.x / a.tiles_x) * a.TH, tw0 = (blockIdx.x % a.tiles_x) * a.TW;
+    const uint32_t cgi = window_div(wave, a.pg, a.mPg), pgi = wave - cgi * a.pg;
+    const uint32_t tile_y = window_div(blockIdx.x, a.tiles_x, a.mTilesX);
+    const uint32_t th0 = tile_y * a.TH, tw0 = (blockIdx.x - tile_y * a.tiles_x) * a.TW;
     const uint32_t grp = blockIdx.y * a.cg + cgi;                    // block of output channels of this wave
     const uint32_t co0 = grp * ct;
     const uint32_t bz = blockIdx.z * BT;
@@ -248,7 +249,7 @@ void conv2d_rbm_kernel(const int4 *__restrict__ sets, const uint32_t *__restrict
     const uint32_t pl = pgi * PPW + lane / LPP, b4 = lane % LPP;
     const bool pvalid = pl < a.TH * a.TW;
     const uint32_t pc = window_slot_pixel(a, pl & 63u);          // slots beyond the tile repeat a pixel of their group
-    const uint32_t ty = pc / a.TW, tx = pc % a.TW;
+    const uint32_t ty = window_div(pc, a.TW, a.mTW), tx = pc - ty * a.TW;
     const bool live = computes && pvalid && th0 + ty < g.H_out && tw0 + tx < g.W_out;
     const uint32_t lanebase = ((ty * a.sth * a.IW + tx * a.stw) << SHIFT) + b4 * 16u;   // bytes
     const uint32_t buf_bytes = a.buf_f4 * 16u;
@@ -263,7 +264,8 @@ void conv2d_rbm_kernel(const int4 *__restrict__ sets, const uint32_t *__restrict
         gcl[k] = 0xffffffffu;
         if (e < a.win_f4) {
             const uint32_t eb = e % LPP, px = e / LPP;
-            const uint32_t iw = px % a.IW, rest = px / a.IW, ih = rest % a.IH, cl = rest / a.IH;
+            const uint32_t rest = window_div(px, a.IW, a.mIW), iw = px - rest * a.IW;
+            const uint32_t cl = window_div(rest, a.IH, a.mIH), ih = rest - cl * a.IH;
             const int32_t gh = (int32_t)(th0 * g.stride_h + ih * a.sbh) - (int32_t)g.pad_h;
             const int32_t gw = (int32_t)(tw0 * g.stride_w + iw * a.sbw) - (int32_t)g.pad_w;
             gcl[k] = cl;
@@ -553,6 +555,8 @@ so_status so_conv_rbm_launch(so_ctx *ctx, const so_conv_plan *plan, const float 
     a.sth = window_step(plan->g.kH, plan->g.stride_h); a.stw = window_step(plan->g.kW, plan->g.stride_w);
     a.sbh = window_subsample(plan->g.kH, plan->g.stride_h); a.sbw = window_subsample(plan->g.kW, plan->g.stride_w);
     window_pixel_order(a, LPP);
+    a.mIW = window_magic(a.IW); a.mIH = window_magic(a.IH); a.mTW = window_magic(a.TW);
+    a.mTilesX = window_magic(a.tiles_x); a.mPg = window_magic(a.pg);
     a.ws = so_lds::wait_status{0, nullptr};      // this kernel synchronises with barriers
     const size_t lds = (size_t)a.nbuf * a.buf_f4 * 16;
     // a layout whose chunks were sized for a smaller batch tile than this batch's does not fit
