@@ -744,6 +744,8 @@ so_status build_window(so_ctx *ctx, so_conv_plan *plan, const std::vector<uint32
     w.tiles_y = so_ceil_div(g.H_out, w.TH);
     w.tiles_x = so_ceil_div(g.W_out, w.TW);
     if ((uint64_t)w.IH * w.IW > 4096) return SO_OK;
+    // the kernels turn a workgroup's index into its tile with window_div: index * tiles_x must fit 32 bits
+    if ((uint64_t)w.tiles_x * w.tiles_x * w.tiles_y >= (1ull << 32)) return SO_OK;
     // Channel chunk: two windows (plus their zero planes) fit LDS, one window fits the copy loop.
     // Both depend on the batch tile (16, 8 or 4 entries): a smaller tile lets a chunk hold more
     // channels, i.e. fewer chunks, fewer barriers and longer runs -- what small batches, whose
