@@ -84,7 +84,7 @@ __device__ __forceinline__ void steps8_v3(const char *lds, uint32_t base, u32x2 
 // MODE 0/1/2: 8 ds_read_b128 / b64 / b32 per iteration (inline asm, so that none is merged or hoisted),
 //             each lane its own 16 / 8 / 4 bytes (consecutive lanes, consecutive addresses: no bank
 //             conflict), results never used.
-// MODE 18:    8 ds_write_b128 per iteration.
+// MODE 18/20/21: 8 ds_write_b128 / b64 / b32 per iteration.
 // MODE 19:    8 ds_read_b128 per iteration, every lane at an address of its own (bank-conflict patterns).
 // MODE 3:     32 independent v_fma_f32 per iteration, no memory access.
 // MODE 4:     32 v_fmac_f32_dpp row_newbcast per iteration (the multiply-add of the LDS-fed kernels' steps).
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(kThreads) void probe(float *out, unsigned long long
     float r[32];
 #pragma unroll
     for (int j = 0; j < 32; ++j) r[j] = (float)(tid + j);
-    const uint32_t addr = (tid & 63u) * ((MODE == 0 || MODE == 18) ? 16u : MODE == 1 ? 8u : 4u) + (tid >> 6) * 4096u;
+    const uint32_t addr = (tid & 63u) * ((MODE == 0 || MODE == 18) ? 16u : (MODE == 1 || MODE == 20) ? 8u : 4u) + (tid >> 6) * 4096u;
     float a4[4] = {0.f, 0.f, 0.f, 0.f};
     const uint32_t eo = offs[tid & 63u];                  // per-lane step offsets (multiples of 256 below 16 KB)
     const float ew = 1.0f + (float)(tid & 15u);
@@ -146,6 +146,26 @@ __global__ __launch_bounds__(kThreads) void probe(float *out, unsigned long long
             asm volatile("ds_write_b128 %0, %1\n\tds_write_b128 %0, %1 offset:1024\n\tds_write_b128 %0, %1 offset:2048\n\t"
                          "ds_write_b128 %0, %1 offset:3072\n\tds_write_b128 %0, %1\n\tds_write_b128 %0, %1 offset:1024\n\t"
                          "ds_write_b128 %0, %1 offset:2048\n\tds_write_b128 %0, %1 offset:3072\n\ts_waitcnt lgkmcnt(0)"
+                         : : "v"(addr), "v"(v) : "memory");
+        } else if constexpr (MODE == 22) {
+            // the same with every write of an iteration at another address (8 KB per wave)
+            f32x4 v = {1.f, 2.f, 3.f, (float)it};
+            const uint32_t a8 = (tid & 63u) * 16u + (tid >> 6) * 8192u;
+            asm volatile("ds_write_b128 %0, %1\n\tds_write_b128 %0, %1 offset:1024\n\tds_write_b128 %0, %1 offset:2048\n\t"
+                         "ds_write_b128 %0, %1 offset:3072\n\tds_write_b128 %0, %1 offset:4096\n\tds_write_b128 %0, %1 offset:5120\n\t"
+                         "ds_write_b128 %0, %1 offset:6144\n\tds_write_b128 %0, %1 offset:7168\n\ts_waitcnt lgkmcnt(0)"
+                         : : "v"(a8), "v"(v) : "memory");
+        } else if constexpr (MODE == 20) {
+            f32x2 v = {1.f, (float)it};
+            asm volatile("ds_write_b64 %0, %1\n\tds_write_b64 %0, %1 offset:512\n\tds_write_b64 %0, %1 offset:1024\n\t"
+                         "ds_write_b64 %0, %1 offset:1536\n\tds_write_b64 %0, %1\n\tds_write_b64 %0, %1 offset:512\n\t"
+                         "ds_write_b64 %0, %1 offset:1024\n\tds_write_b64 %0, %1 offset:1536\n\ts_waitcnt lgkmcnt(0)"
+                         : : "v"(addr), "v"(v) : "memory");
+        } else if constexpr (MODE == 21) {
+            float v = (float)it;
+            asm volatile("ds_write_b32 %0, %1\n\tds_write_b32 %0, %1 offset:256\n\tds_write_b32 %0, %1 offset:512\n\t"
+                         "ds_write_b32 %0, %1 offset:768\n\tds_write_b32 %0, %1\n\tds_write_b32 %0, %1 offset:256\n\t"
+                         "ds_write_b32 %0, %1 offset:512\n\tds_write_b32 %0, %1 offset:768\n\ts_waitcnt lgkmcnt(0)"
                          : : "v"(addr), "v"(v) : "memory");
         } else if constexpr (MODE == 3) {
             const float w = (float)it;
@@ -335,6 +355,9 @@ int main()
     for (int waves : {16, 8}) {
         run<0>("ds_read_b128, conflict-free", cus, waves, 8.0 * 64 * 16, "bytes", dOut, dCyc, dOffs, dEnts);
         run<18>("ds_write_b128, conflict-free", cus, waves, 8.0 * 64 * 16, "bytes", dOut, dCyc, dOffs, dEnts);
+        run<22>("ds_write_b128, conflict-free, 8 addresses per lane", cus, waves, 8.0 * 64 * 16, "bytes", dOut, dCyc, dOffs, dEnts);
+        run<20>("ds_write_b64, conflict-free", cus, waves, 8.0 * 64 * 8, "bytes", dOut, dCyc, dOffs, dEnts);
+        run<21>("ds_write_b32, conflict-free", cus, waves, 8.0 * 64 * 4, "bytes", dOut, dCyc, dOffs, dEnts);
         run<1>("ds_read_b64, conflict-free", cus, waves, 8.0 * 64 * 8, "bytes", dOut, dCyc, dOffs, dEnts);
         run<2>("ds_read_b32, conflict-free", cus, waves, 8.0 * 64 * 4, "bytes", dOut, dCyc, dOffs, dEnts);
         run<3>("v_fma_f32, 32 independent chains", cus, waves, 32.0 * 64, "multiply-adds", dOut, dCyc, dOffs, dEnts);
