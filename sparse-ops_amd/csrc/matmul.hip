@@ -200,8 +200,8 @@ void launch_act(so_ctx *ctx, const so_ellpack *E, const float *dX, uint32_t C, c
 // can keep in flight are bounded by its registers.  Here a workgroup of 16 waves
 // shares one (row, 64-column tile): the waves split the row's nonzeros among them
 // for the gathers (16 times the loads in flight), park the gathered X segments in
-// LDS in slot order, and the first wave then runs the multiply-adds over them in
-// slot order starting from the bias -- the same rounding sequence as the row kernel.
+// LDS, and the first wave then runs the multiply-adds over them in slot order
+// starting from the bias -- the same rounding sequence as the row kernel.
 // ---------------------------------------------------------------------------
 
 constexpr int kShareWaves = 16;
@@ -217,8 +217,8 @@ void ellpack_matmul_shared_gather_kernel(const float *__restrict__ Wd, const uin
                                          const float *__restrict__ bias, float *__restrict__ Y, uint32_t ntiles)
 {
     extern __shared__ __attribute__((aligned(16))) float share_lds[];
-    float *xs = share_lds;                              // [kShareChunk][64]
-    float *ws = share_lds + (size_t)kShareChunk * 64;   // [kShareChunk]
+    float4 *xs4 = reinterpret_cast<float4 *>(share_lds);   // [kShareChunk / 4][64 lanes][4 slots]
+    float *ws = share_lds + (size_t)kShareChunk * 64;      // [kShareChunk]
     const uint32_t tile = blockIdx.x % ntiles, row = blockIdx.x / ntiles;   // the grid is exactly m * ntiles
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -242,21 +242,25 @@ void ellpack_matmul_shared_gather_kernel(const float *__restrict__ Wd, const uin
                 x[u] = xcol[(size_t)irow[j] * C];
             }
             if (lane < mine) ws[w0 + lane] = wrow[s0 + w0 + lane];
+            // four consecutive slots of a lane side by side: the wave that multiplies takes them with one read
 #pragma unroll
-            for (int u = 0; u < kSharePerWave; ++u)
-                if ((uint32_t)u < mine) xs[(w0 + u) * 64u + lane] = x[u];
+            for (int u = 0; u < kSharePerWave; u += 4)
+                if ((uint32_t)u < mine) xs4[((w0 + u) / 4u) * 64u + lane] = make_float4(x[u], x[u + 1], x[u + 2], x[u + 3]);
         }
         __syncthreads();
         if (wave == 0) {
+            // One wave, one instruction at a time: what counts is instructions per slot -- a 16-byte read of four
+            // weights (every lane the same address), one of this lane's four operands, four multiply-adds.
             uint32_t s = 0;
             for (; s + 8 <= chunk; s += 8) {
-                float w[8], x[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) { w[u] = ws[s + u]; x[u] = xs[(s + u) * 64u + lane]; }
-#pragma unroll
-                for (int u = 0; u < 8; ++u) acc = __builtin_fmaf(w[u], x[u], acc);
+                const float4 wa = *reinterpret_cast<const float4 *>(ws + s), wb = *reinterpret_cast<const float4 *>(ws + s + 4);
+                const float4 xa = xs4[(s / 4u) * 64u + lane], xb = xs4[(s / 4u + 1u) * 64u + lane];
+                acc = __builtin_fmaf(wa.x, xa.x, acc); acc = __builtin_fmaf(wa.y, xa.y, acc);
+                acc = __builtin_fmaf(wa.z, xa.z, acc); acc = __builtin_fmaf(wa.w, xa.w, acc);
+                acc = __builtin_fmaf(wb.x, xb.x, acc); acc = __builtin_fmaf(wb.y, xb.y, acc);
+                acc = __builtin_fmaf(wb.z, xb.z, acc); acc = __builtin_fmaf(wb.w, xb.w, acc);
             }
-            for (; s < chunk; ++s) acc = __builtin_fmaf(ws[s], xs[s * 64u + lane], acc);
+            for (; s < chunk; ++s) acc = __builtin_fmaf(ws[s], share_lds[(s / 4u) * 256u + lane * 4u + (s & 3u)], acc);
         }
         __syncthreads();                                  // the next chunk overwrites what wave 0 was reading
     }
