@@ -87,6 +87,7 @@ __device__ __forceinline__ void steps8_v3(const char *lds, uint32_t base, u32x2 
 // MODE 18/20/21: 8 ds_write_b128 / b64 / b32 per iteration.
 // MODE 19:    8 ds_read_b128 per iteration, every lane at an address of its own (bank-conflict patterns).
 // MODE 3:     32 independent v_fma_f32 per iteration, no memory access.
+// MODE 23:    32 v_fmac_f32 per iteration on one accumulator (a dependent chain).
 // MODE 4:     32 v_fmac_f32_dpp row_newbcast per iteration (the multiply-add of the LDS-fed kernels' steps).
 // MODE 5:     the step loop of the tiled matmul and the windowed convolution itself (csrc/dpp_steps.h):
 //             16 steps per iteration, each one ds_read_b128 + one address add + four multiply-adds.
@@ -178,6 +179,11 @@ __global__ __launch_bounds__(kThreads) void probe(float *out, unsigned long long
             for (int j = 0; j < 16; ++j) r[j] = __builtin_fmaf(wv, r[16 + j], r[j]);
 #pragma unroll
             for (int j = 0; j < 16; ++j) r[j] = __builtin_fmaf(wv, r[31 - j], r[j]);
+        } else if constexpr (MODE == 23) {
+            // one chain: every multiply-add waits for the one before it
+            const float wv = 1.0f + 1e-7f * (float)it;
+#pragma unroll
+            for (int j = 0; j < 32; ++j) asm volatile("v_fmac_f32 %0, %1, %2" : "+v"(r[0]) : "v"(wv), "v"(r[1 + (j & 15)]));
         } else if constexpr (MODE == 4) {
 #pragma unroll
             for (int j = 0; j < 32; ++j)
@@ -352,6 +358,10 @@ int main()
         for (int i = 0; i < 64; ++i) offs[i] = (uint32_t)((i * 37) % 60) * 256u;
         CK(hipMemcpy(dOffs, offs.data(), 256, hipMemcpyHostToDevice));
     }
+    // one wave per SIMD, one chain: 256 multiply-adds per CU in flight, so clocks from one multiply-add to the next that
+    // uses its result = 256 / the rate printed
+    run<23>("v_fmac_f32, one dependent chain per lane", cus, 4, 32.0 * 64, "multiply-adds", dOut, dCyc, dOffs, dEnts);
+    run<23>("v_fmac_f32, one dependent chain per lane", cus, 8, 32.0 * 64, "multiply-adds", dOut, dCyc, dOffs, dEnts);
     for (int waves : {16, 8}) {
         run<0>("ds_read_b128, conflict-free", cus, waves, 8.0 * 64 * 16, "bytes", dOut, dCyc, dOffs, dEnts);
         run<18>("ds_write_b128, conflict-free", cus, waves, 8.0 * 64 * 16, "bytes", dOut, dCyc, dOffs, dEnts);
